@@ -1,0 +1,181 @@
+"""Pins for the CPU oracle.  Each check is chosen so that a plausible mistake (a
+dropped sink term, a wrong GQA head map, a transposed stride, scale applied twice,
+masking off by one) fails at least one of them."""
+import math
+
+import pytest
+import torch
+
+from flash_attention_factory_amd import workloads as W
+from _torch_ref import brute_force, call_oracle, sdpa_reference
+
+
+def _grid_case(**kw):
+    base = dict(batch_size=2, nheads=8, nheads_k=2, d=64, seqlen_k=339, varlen=True, has_sinks=False)
+    base.update(kw)
+    return W.make_test_shaped(**base)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(),
+    dict(has_sinks=True),
+    dict(d=128, nheads=10, nheads_k=2, seqlen_k=800),
+    dict(d=128, nheads=2, nheads_k=2, seqlen_k=128, varlen=False, has_sinks=True),
+    dict(fp8=True, nheads=14, nheads_k=2, seqlen_k=799, has_sinks=True),
+    dict(layout=W.HEAD_MAJOR, block_size=16, seqlen_k=257),
+    dict(dtype=torch.bfloat16, fp8=True, d=128, seqlen_k=1024, has_sinks=True),
+])
+def test_attention_ref_equals_sdpa(oracle, kw):
+    w = _grid_case(**kw)
+    _, got = call_oracle(oracle.attention_ref, w, want_f32=True)
+    want = sdpa_reference(w)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("index", [0, 1, 3])
+def test_attention_ref_on_measured_configs(oracle, index):
+    w = W.make_config(index, num_seqs=2, pool_blocks=384)
+    _, got = call_oracle(oracle.attention_ref, w, want_f32=True)
+    torch.testing.assert_close(got, sdpa_reference(w), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("sinks", [False, True])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_attention_ref_brute_force_float64(oracle, sinks, fp8):
+    w = W.make_test_shaped(batch_size=2, nheads=4, nheads_k=2, d=8, seqlen_k=9, varlen=True,
+                           has_sinks=sinks, fp8=fp8, block_size=4, seed=3)
+    if sinks:
+        w.sinks = torch.tensor([0.5, -1.0, 2.0, 0.0], dtype=torch.float16)
+    _, got = call_oracle(oracle.attention_ref, w, want_f32=True)
+    torch.testing.assert_close(got.double(), brute_force(w), rtol=1e-5, atol=1e-6)
+
+
+def test_closed_forms(oracle):
+    w = _grid_case(d=64, nheads=4, nheads_k=2, seqlen_k=70, varlen=False, block_size=16, layout=W.HEAD_MAJOR)
+    S, H, D = w.query.shape
+    # ctx = 1: out is the first value row of the head's kv head
+    w1 = W.Workload(**{**w.__dict__})
+    w1.context_lens = torch.ones(S, dtype=torch.int32)
+    _, got = call_oracle(oracle.attention_ref, w1, want_f32=True)
+    for s in range(S):
+        for h in range(H):
+            v0 = w.value_cache[int(w.block_tables[s, 0]), h // 2, 0].float()
+            torch.testing.assert_close(got[s, h], v0, rtol=0, atol=0)
+    # ctx = 1 with a sink: v0 / (1 + exp(sink - s0))
+    w1.sinks = torch.tensor([0.25, 1.5, -0.75, 3.0], dtype=torch.float16)
+    _, got = call_oracle(oracle.attention_ref, w1, want_f32=True)
+    for s in range(S):
+        for h in range(H):
+            blk = int(w.block_tables[s, 0])
+            s0 = float((w.query[s, h].float() * w.scale) @ w.key_cache[blk, h // 2, 0].float())
+            v0 = w.value_cache[blk, h // 2, 0].float()
+            want = v0 / (1.0 + math.exp(float(w1.sinks[h]) - s0))
+            torch.testing.assert_close(got[s, h], want, rtol=1e-5, atol=1e-7)
+    # q = 0: uniform weights -> mean of the first ctx value rows
+    w2 = W.Workload(**{**w.__dict__})
+    w2.query = torch.zeros_like(w.query)
+    w2.context_lens = torch.tensor([37, 70], dtype=torch.int32)
+    _, got = call_oracle(oracle.attention_ref, w2, want_f32=True)
+    for s in range(S):
+        n = int(w2.context_lens[s])
+        rows = torch.stack([w.value_cache[int(w.block_tables[s, t // 16]), 1, t % 16].float() for t in range(n)])
+        torch.testing.assert_close(got[s, 3], rows.mean(0), rtol=1e-5, atol=1e-6)
+    # V = const c and a sink: out = c * (1 - w_sink); all K rows equal -> w_sink known
+    w3 = W.Workload(**{**w.__dict__})
+    w3.value_cache = torch.full_like(w.value_cache, 0.5)
+    w3.key_cache = torch.zeros_like(w.key_cache)
+    w3.sinks = torch.tensor([1.0, 1.0, 1.0, 1.0], dtype=torch.float16)
+    _, got = call_oracle(oracle.attention_ref, w3, want_f32=True)
+    want = 0.5 * 70.0 / (70.0 + math.e)
+    torch.testing.assert_close(got, torch.full_like(got, want), rtol=1e-5, atol=1e-7)
+
+
+def test_invariants(oracle):
+    w = _grid_case(d=64, nheads=8, nheads_k=2, seqlen_k=300, has_sinks=True)
+    base = call_oracle(oracle.attention_ref, w)
+    # permuting pool blocks together with the table changes nothing
+    NB = w.key_cache.shape[0]
+    perm = torch.randperm(NB, generator=torch.Generator().manual_seed(5))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(NB)
+    w2 = W.Workload(**{**w.__dict__})
+    w2.key_cache = w.key_cache[perm].contiguous()
+    w2.value_cache = w.value_cache[perm].contiguous()
+    w2.block_tables = inv[w.block_tables.long()].to(torch.int32)
+    assert torch.equal(call_oracle(oracle.attention_ref, w2), base)
+    # rows past context_len never matter: poison them with NaN
+    w3 = W.Workload(**{**w.__dict__})
+    kc, vc = w.key_cache.clone(), w.value_cache.clone()
+    for s in range(w.num_seqs):
+        n = int(w.context_lens[s])
+        for t in range(n, w.block_tables.shape[1] * w.block_size):
+            blk = int(w.block_tables[s, t // w.block_size])
+            kc[blk, t % w.block_size] = float("nan")
+            vc[blk, t % w.block_size] = float("nan")
+    w3.key_cache, w3.value_cache = kc, vc
+    assert torch.equal(call_oracle(oracle.attention_ref, w3), base)
+    # sink = -inf is "no sink" (that is how the upstream kernel encodes it,
+    # paged_attention_kernel_loop.hpp:186-189)
+    w4 = W.Workload(**{**w.__dict__})
+    w4.sinks = torch.full_like(w.sinks, float("-inf"))
+    w5 = W.Workload(**{**w.__dict__})
+    w5.sinks = None
+    assert torch.equal(call_oracle(oracle.attention_ref, w4), call_oracle(oracle.attention_ref, w5))
+    # query heads of one group with identical q rows give identical outputs
+    w6 = W.Workload(**{**w.__dict__})
+    q = w.query.clone()
+    q[:, 1] = q[:, 0]
+    w6.query = q
+    w6.sinks = None
+    o = call_oracle(oracle.attention_ref, w6)
+    assert torch.equal(o[:, 0], o[:, 1])
+    # both cache layouts describe the same pool
+    w7 = W.Workload(**{**w.__dict__})
+    w7.key_cache = w.key_cache.permute(0, 2, 1, 3).contiguous()
+    w7.value_cache = w.value_cache.permute(0, 2, 1, 3).contiguous()
+    w7.layout = W.HEAD_MAJOR
+    assert torch.equal(call_oracle(oracle.attention_ref, w7), base)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(d=128, nheads=8, nheads_k=1, seqlen_k=2048, has_sinks=True),
+    dict(d=64, nheads=6, nheads_k=2, seqlen_k=799),
+    dict(d=128, nheads=16, nheads_k=2, seqlen_k=1024, fp8=True, has_sinks=True),
+])
+def test_kernel_models_track_attention_ref(oracle, kw):
+    """The kernel-arithmetic restatement differs from the reference only by where it
+    rounds (probabilities to 16 bit, scale after the dot), so it must sit within a few
+    16-bit ulps of it; and loop == partition + reduce by split-invariance of log-sum-exp."""
+    w = _grid_case(**kw)
+    _, ref = call_oracle(oracle.attention_ref, w, want_f32=True)
+    _, loop = call_oracle(oracle.kernel_loop, w, partition_size=w.partition_size, want_f32=True)
+    NP = w.max_num_partitions + 2  # padding slots must not be read
+    es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=w.partition_size,
+                              max_num_partitions=NP)
+    _, red = oracle.kernel_reduce(es, ml, tmp, w.context_lens, partition_size=w.partition_size,
+                                  q_dtype=w.query.dtype, want_f32=True)
+    scale = ref.abs().max().item()
+    assert (loop - ref).abs().max().item() <= 2e-3 * scale
+    assert (red - ref).abs().max().item() <= 2e-3 * scale
+    assert (red - loop).abs().max().item() <= 2e-3 * scale
+    # scratch semantics: live slots finite, dead slots untouched
+    for s in range(w.num_seqs):
+        live = math.ceil(int(w.context_lens[s]) / w.partition_size)
+        assert torch.isfinite(es[s, :, :live]).all() and torch.isnan(es[s, :, live:]).all()
+        assert torch.isnan(tmp[s, :, live:]).all()
+
+
+def test_partition_scratch_closed_form(oracle):
+    """One partition, no sink: max_logits is the largest logit, exp_sums is
+    sum exp(s - max), tmp_out is the normalised output itself."""
+    w = _grid_case(d=64, nheads=4, nheads_k=2, seqlen_k=200, varlen=False)
+    es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=256, max_num_partitions=1)
+    _, ref = call_oracle(oracle.attention_ref, w, want_f32=True)
+    assert (tmp[:, :, 0] - ref).abs().max().item() <= 2e-3 * ref.abs().max().item()
+    from _torch_ref import dense_kv
+    k = dense_kv(w, w.key_cache)  # [S, T, Hk, D]
+    for s in range(w.num_seqs):
+        for h in range(w.num_heads):
+            logits = (k[s, :, h // 2] @ w.query[s, h].float()) * w.scale
+            torch.testing.assert_close(ml[s, h, 0], logits.max(), rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(es[s, h, 0], torch.exp(logits - logits.max()).sum(), rtol=1e-5, atol=1e-6)
