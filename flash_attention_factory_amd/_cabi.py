@@ -1,0 +1,104 @@
+"""ctypes binding of libfa_paged_attention.so (declarations: include/fa_paged_attention.h).
+
+There is no fallback: if the HIP library is missing or a call fails, this raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIBRARY = os.path.join(_PKG, "libfa_paged_attention.so")
+
+FA_OK = 0
+FA_ERR_NULL_POINTER = 1
+FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE = 2
+FA_ERR_UNSUPPORTED_GROUP = 3
+FA_ERR_UNSUPPORTED_DTYPE = 4
+FA_ERR_PARTITION_OVERFLOW = 5
+FA_ERR_BAD_SHAPE = 6
+FA_ERR_RUNTIME = 7
+
+FA_DTYPE_F16 = 0
+FA_DTYPE_BF16 = 1
+
+EXPORTS = (
+    "fa_paged_attention_loop",
+    "fa_paged_attention_reduce",
+    "fa_paged_attention_fp8_loop",
+    "fa_paged_attention_fp8_reduce",
+    "fa_last_error",
+    "fa_paged_attention_abi_version",
+)
+
+
+class Shape(ctypes.Structure):
+    _fields_ = [
+        ("num_seqs", ctypes.c_int32),
+        ("num_heads", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_size", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+        ("max_blocks_per_seq", ctypes.c_int32),
+        ("max_num_partitions", ctypes.c_int32),
+        ("partition_size", ctypes.c_int32),
+        ("kv_block_stride", ctypes.c_int64),
+        ("kv_token_stride", ctypes.c_int64),
+        ("kv_head_stride", ctypes.c_int64),
+        ("q_dtype", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class Options(ctypes.Structure):
+    _fields_ = [
+        ("sinks", ctypes.c_void_p),
+        ("alibi_slopes", ctypes.c_void_p),
+        ("softcap", ctypes.c_float),
+        ("fp8_scale", ctypes.c_float),
+        ("stream", ctypes.c_void_p),
+        ("elapsed_us", ctypes.POINTER(ctypes.c_float)),
+        ("validate_only", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class PagedAttentionError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[fa_status {code}] {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the in-tree HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIBRARY):
+        raise RuntimeError(
+            f"{LIBRARY} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(there is no CPU or PyTorch fallback for the paged-attention kernels)")
+    L = ctypes.CDLL(LIBRARY)
+    P = ctypes.c_void_p
+    common = [P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32]
+    tail = [ctypes.POINTER(Shape), ctypes.POINTER(Options)]
+    for name in ("fa_paged_attention_loop", "fa_paged_attention_fp8_loop"):
+        fn = getattr(L, name)
+        fn.argtypes = common + tail
+        fn.restype = ctypes.c_int32
+    for name in ("fa_paged_attention_reduce", "fa_paged_attention_fp8_reduce"):
+        fn = getattr(L, name)
+        fn.argtypes = common + [P, P, P] + tail
+        fn.restype = ctypes.c_int32
+    L.fa_last_error.restype = ctypes.c_char_p
+    L.fa_paged_attention_abi_version.restype = ctypes.c_int32
+    _lib = L
+    return L
+
+
+def check(code: int) -> None:
+    if code != FA_OK:
+        raise PagedAttentionError(code, load().fa_last_error().decode())

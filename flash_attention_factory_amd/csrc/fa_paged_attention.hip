@@ -1,0 +1,61 @@
+// extern "C" surface of libfa_paged_attention.so: four entry points, one per host
+// launcher, declared in include/fa_paged_attention.h.
+#include "../../include/fa_paged_attention.h"
+
+#include "launch_kernels_fp8_loop.h"
+#include "launch_kernels_fp8_reduce.h"
+#include "launch_kernels_loop.h"
+#include "launch_kernels_reduce.h"
+
+#define FA_EXPORT extern "C" __attribute__((visibility("default")))
+
+FA_EXPORT int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_cache,
+                                          const void *value_cache, const int32_t *block_tables,
+                                          const int32_t *context_lens, float scale,
+                                          int32_t max_context_len,
+                                          const fa_paged_attention_shape *shape,
+                                          const fa_paged_attention_options *options) {
+  return fa::dispatch_paged_attention_loop(out, query, key_cache, value_cache, block_tables,
+                                           context_lens, scale, max_context_len, shape, options);
+}
+
+FA_EXPORT int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
+                                            const void *value_cache, const int32_t *block_tables,
+                                            const int32_t *context_lens, float scale,
+                                            int32_t max_context_len, float *exp_sums,
+                                            float *max_logits, float *tmp_out,
+                                            const fa_paged_attention_shape *shape,
+                                            const fa_paged_attention_options *options) {
+  return fa::dispatch_paged_attention(out, query, key_cache, value_cache, block_tables,
+                                      context_lens, scale, max_context_len, exp_sums, max_logits,
+                                      tmp_out, shape, options);
+}
+
+FA_EXPORT int32_t fa_paged_attention_fp8_loop(void *out, const void *query, const void *key_cache,
+                                              const void *value_cache,
+                                              const int32_t *block_tables,
+                                              const int32_t *context_lens, float scale,
+                                              int32_t max_context_len,
+                                              const fa_paged_attention_shape *shape,
+                                              const fa_paged_attention_options *options) {
+  return fa::dispatch_paged_attention_fp8_loop(out, query, key_cache, value_cache, block_tables,
+                                               context_lens, scale, max_context_len, shape,
+                                               options);
+}
+
+FA_EXPORT int32_t fa_paged_attention_fp8_reduce(void *out, const void *query,
+                                                const void *key_cache, const void *value_cache,
+                                                const int32_t *block_tables,
+                                                const int32_t *context_lens, float scale,
+                                                int32_t max_context_len, float *exp_sums,
+                                                float *max_logits, float *tmp_out,
+                                                const fa_paged_attention_shape *shape,
+                                                const fa_paged_attention_options *options) {
+  return fa::dispatch_paged_attention_fp8(out, query, key_cache, value_cache, block_tables,
+                                          context_lens, scale, max_context_len, exp_sums,
+                                          max_logits, tmp_out, shape, options);
+}
+
+FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
+
+FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 1; }

@@ -1,0 +1,205 @@
+// Host-side pieces shared by the four launchers: error text, argument checks,
+// kernel-parameter assembly and event timing.
+//
+// Upstream has no counterpart for the checks (paged_attention_loop.cpp:44-65 reads
+// pointers and sizes without looking at them) and reports errors by throwing
+// std::runtime_error from the dispatchers (launch_kernels_loop.h:114-115,170-172);
+// here the same conditions become status codes because nothing may throw across a C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/fa_paged_attention.h"
+#include "paged_attention_kernel.h"
+#include "paged_attention_policy.h"
+#include "paged_attention_reduce_kernel.h"
+
+namespace fa {
+
+inline char *error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+inline fa_status fail(fa_status code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define FA_HIP_CHECK(expr)                                                                  \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      return ::fa::fail(FA_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(e_));     \
+  } while (0)
+
+inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+inline int ilog2(int32_t v) {
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
+struct Resolved {
+  int32_t group;
+  int32_t partition_size;
+  int32_t kv_elem_bytes;
+  float fp8_scale;
+  hipStream_t stream;
+  float *elapsed_us;
+  bool validate_only;
+  const void *sinks;
+};
+
+// Checks every argument the kernels rely on.  `kv8` selects byte caches, `split`
+// the presence of the scratch arrays.
+inline fa_status validate_and_resolve(const void *out, const void *query, const void *key_cache,
+                                      const void *value_cache, const int32_t *block_tables,
+                                      const int32_t *context_lens, int32_t max_context_len,
+                                      const float *exp_sums, const float *max_logits,
+                                      const float *tmp_out, const fa_paged_attention_shape *s,
+                                      const fa_paged_attention_options *o, bool kv8, bool split,
+                                      Resolved *r) {
+  error_buffer()[0] = 0;
+  if (!s) return fail(FA_ERR_NULL_POINTER, "shape is NULL");
+  if (!out || !query || !key_cache || !value_cache || !block_tables || !context_lens)
+    return fail(FA_ERR_NULL_POINTER, "out, query, key_cache, value_cache, block_tables and "
+                                     "context_lens must all be non-NULL");
+  if (split && (!exp_sums || !max_logits || !tmp_out))
+    return fail(FA_ERR_NULL_POINTER, "exp_sums, max_logits and tmp_out must be non-NULL");
+  if (s->q_dtype != FA_DTYPE_F16 && s->q_dtype != FA_DTYPE_BF16)
+    return fail(FA_ERR_UNSUPPORTED_DTYPE, "q_dtype %d is neither fp16 (0) nor bf16 (1)", s->q_dtype);
+  if ((s->head_size != 64 && s->head_size != 128) || s->block_size < 16 || !is_pow2(s->block_size))
+    return fail(FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE,
+                "Unsupported head size or block size (head_size %d must be 64 or 128, block_size "
+                "%d a power of two >= 16)", s->head_size, s->block_size);
+  if (s->num_seqs <= 0 || s->num_heads <= 0 || s->num_kv_heads <= 0 || s->max_blocks_per_seq <= 0)
+    return fail(FA_ERR_BAD_SHAPE, "num_seqs, num_heads, num_kv_heads and max_blocks_per_seq must be positive");
+  if (s->num_seqs > 65535)
+    return fail(FA_ERR_BAD_SHAPE, "num_seqs %d exceeds the grid limit 65535", s->num_seqs);
+  if (s->num_heads % s->num_kv_heads != 0)
+    return fail(FA_ERR_UNSUPPORTED_GROUP, "Unsupported number of queries per token: num_heads %d is "
+                                          "not a multiple of num_kv_heads %d", s->num_heads, s->num_kv_heads);
+  r->group = s->num_heads / s->num_kv_heads;
+  if (r->group > kMaxGroup)
+    return fail(FA_ERR_UNSUPPORTED_GROUP, "Unsupported number of queries per token: %d (at most %d)",
+                r->group, kMaxGroup);
+  r->kv_elem_bytes = kv8 ? 1 : 2;
+  const int64_t eb = r->kv_elem_bytes;
+  if (s->kv_block_stride <= 0 || s->kv_token_stride <= 0 || s->kv_head_stride <= 0)
+    return fail(FA_ERR_BAD_SHAPE, "kv strides must be positive");
+  if ((s->kv_block_stride * eb) % 16 || (s->kv_token_stride * eb) % 16 || (s->kv_head_stride * eb) % 16)
+    return fail(FA_ERR_BAD_SHAPE, "kv strides must be multiples of 16 bytes");
+  if (s->kv_token_stride < s->head_size || s->kv_head_stride < s->head_size)
+    return fail(FA_ERR_BAD_SHAPE, "kv_token_stride and kv_head_stride must each cover one head_size row");
+  if (((uintptr_t)key_cache | (uintptr_t)value_cache | (uintptr_t)query | (uintptr_t)out) % 16)
+    return fail(FA_ERR_BAD_SHAPE, "out, query, key_cache and value_cache must be 16-byte aligned");
+  r->partition_size = s->partition_size > 0 ? s->partition_size : default_partition_size(s->head_size);
+  if (split) {
+    if (r->partition_size % kChunkTokens)
+      return fail(FA_ERR_BAD_SHAPE, "partition_size %d must be a multiple of %d", r->partition_size, kChunkTokens);
+    if (s->max_num_partitions <= 0 || s->max_num_partitions > 65535)
+      return fail(FA_ERR_BAD_SHAPE, "max_num_partitions %d must be in [1, 65535]", s->max_num_partitions);
+    if (max_context_len > 0 &&
+        (int64_t)s->max_num_partitions * r->partition_size < (int64_t)max_context_len)
+      return fail(FA_ERR_PARTITION_OVERFLOW, "max_context_len %d needs %d partitions of %d tokens, scratch has %d",
+                  max_context_len, (max_context_len + r->partition_size - 1) / r->partition_size,
+                  r->partition_size, s->max_num_partitions);
+    if ((uintptr_t)tmp_out % 16) return fail(FA_ERR_BAD_SHAPE, "tmp_out must be 16-byte aligned");
+  }
+  if (max_context_len > 0 &&
+      (int64_t)s->max_blocks_per_seq * s->block_size < (int64_t)max_context_len)
+    return fail(FA_ERR_BAD_SHAPE, "max_context_len %d does not fit %d blocks of %d tokens", max_context_len,
+                s->max_blocks_per_seq, s->block_size);
+  r->fp8_scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
+  r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
+  r->elapsed_us = o ? o->elapsed_us : nullptr;
+  r->validate_only = o && o->validate_only != 0;
+  r->sinks = o ? o->sinks : nullptr;
+  return FA_OK;
+}
+
+inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits, const void *query,
+                                   const void *key_cache, const void *value_cache,
+                                   const int32_t *block_tables, const int32_t *context_lens,
+                                   float scale, const fa_paged_attention_shape &s, const Resolved &r) {
+  PagedAttnParams p;
+  p.out = out;
+  p.exp_sums = exp_sums;
+  p.max_logits = max_logits;
+  p.query = query;
+  p.key_cache = reinterpret_cast<const char *>(key_cache);
+  p.value_cache = reinterpret_cast<const char *>(value_cache);
+  p.block_tables = block_tables;
+  p.context_lens = context_lens;
+  p.sinks = r.sinks;
+  p.score_scale_log2 = scale * r.fp8_scale * kLog2e;
+  p.out_scale = r.fp8_scale;
+  p.num_heads = s.num_heads;
+  p.group = r.group;
+  p.max_blocks_per_seq = s.max_blocks_per_seq;
+  p.max_num_partitions = s.max_num_partitions;
+  p.partition_size = r.partition_size;
+  p.block_shift = ilog2(s.block_size);
+  p.kv_block_bytes = s.kv_block_stride * r.kv_elem_bytes;
+  p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
+  p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;
+  return p;
+}
+
+// Kernel-only time from a pair of events on the launch stream -- the counterpart of
+// upstream's get_exe_time (launch_kernels_loop.h:6-12), which reads SYCL event
+// profiling info.  Events are created once per thread and device and reused.
+class KernelTimer {
+ public:
+  explicit KernelTimer(bool enabled, hipStream_t stream) : enabled_(enabled), stream_(stream) {}
+  hipError_t start(int slot) {
+    if (!enabled_) return hipSuccess;
+    hipError_t e = ensure();
+    if (e != hipSuccess) return e;
+    return hipEventRecord(events()[2 * slot], stream_);
+  }
+  hipError_t stop(int slot) {
+    if (!enabled_) return hipSuccess;
+    return hipEventRecord(events()[2 * slot + 1], stream_);
+  }
+  hipError_t read(int slot, float *us) {
+    if (!enabled_) return hipSuccess;
+    hipError_t e = hipEventSynchronize(events()[2 * slot + 1]);
+    if (e != hipSuccess) return e;
+    float ms = 0.f;
+    e = hipEventElapsedTime(&ms, events()[2 * slot], events()[2 * slot + 1]);
+    *us = ms * 1000.f;
+    return e;
+  }
+
+ private:
+  static hipEvent_t *events() {
+    static thread_local hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    return ev;
+  }
+  static hipError_t ensure() {
+    static thread_local int device_of_events = -1;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (device_of_events == dev) return hipSuccess;
+    for (int k = 0; k < 4; ++k) {
+      if (events()[k]) (void)hipEventDestroy(events()[k]);
+      e = hipEventCreate(&events()[k]);
+      if (e != hipSuccess) return e;
+    }
+    device_of_events = dev;
+    return hipSuccess;
+  }
+  bool enabled_;
+  hipStream_t stream_;
+};
+
+}  // namespace fa

@@ -1,0 +1,74 @@
+// Host launcher and dispatcher of the single-pass ("loop") paged-attention kernel.
+//
+// Same role and argument list as upstream paged_attention_loop/launch_kernels_loop.h:
+// launch_paged_attn_loop (:16-54) builds the launch geometry and submits one kernel,
+// dispatch_paged_attention_loop (:56-173) maps the runtime (head_size, dtype) onto a
+// template instance.  Block size and query-group size are runtime values here, so the
+// 16-way switch of upstream collapses to head size x dtype.
+#pragma once
+
+#include "launch_common.h"
+
+namespace fa {
+
+// One launch, grid (kv heads, 1, sequences), NW wavefronts per work-group.
+// KV8 selects the E5M2 cache form (used by launch_kernels_fp8_loop.h).
+template <int HEAD_SIZE, typename QT, bool KV8>
+inline fa_status launch_paged_attn_loop(void *out, const void *query, const void *key_cache,
+                                        const void *value_cache, const int32_t *block_tables,
+                                        const int32_t *context_lens, float scale,
+                                        int32_t /*max_context_len: validation only*/,
+                                        const fa_paged_attention_shape &shape, const Resolved &r) {
+  constexpr int NW = WavesPerGroup<false>::value;
+  const PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
+                                        block_tables, context_lens, scale, shape, r);
+  const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+  KernelTimer timer(r.elapsed_us != nullptr, r.stream);
+  FA_HIP_CHECK(timer.start(0));
+  hipLaunchKernelGGL((paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW>), grid, dim3(NW * 64), 0,
+                     r.stream, p);
+  FA_HIP_CHECK(hipGetLastError());
+  FA_HIP_CHECK(timer.stop(0));
+  if (r.elapsed_us) FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
+  return FA_OK;
+}
+
+template <bool KV8>
+inline fa_status dispatch_paged_attention_loop_any(void *out, const void *query,
+                                                   const void *key_cache, const void *value_cache,
+                                                   const int32_t *block_tables,
+                                                   const int32_t *context_lens, float scale,
+                                                   int32_t max_context_len,
+                                                   const fa_paged_attention_shape *shape,
+                                                   const fa_paged_attention_options *options) {
+  Resolved r;
+  fa_status st = validate_and_resolve(out, query, key_cache, value_cache, block_tables, context_lens,
+                                      max_context_len, nullptr, nullptr, nullptr, shape, options,
+                                      KV8, /*split=*/false, &r);
+  if (st != FA_OK || r.validate_only) return st;
+  const bool bf16 = shape->q_dtype == FA_DTYPE_BF16;
+#define FA_LOOP_CASE(HS, QT)                                                                      \
+  return launch_paged_attn_loop<HS, QT, KV8>(out, query, key_cache, value_cache, block_tables,    \
+                                             context_lens, scale, max_context_len, *shape, r)
+  if (shape->head_size == 128) {
+    if (bf16) FA_LOOP_CASE(128, BF16);
+    FA_LOOP_CASE(128, F16);
+  }
+  if (bf16) FA_LOOP_CASE(64, BF16);
+  FA_LOOP_CASE(64, F16);
+#undef FA_LOOP_CASE
+}
+
+inline fa_status dispatch_paged_attention_loop(void *out, const void *query, const void *key_cache,
+                                               const void *value_cache,
+                                               const int32_t *block_tables,
+                                               const int32_t *context_lens, float scale,
+                                               int32_t max_context_len,
+                                               const fa_paged_attention_shape *shape,
+                                               const fa_paged_attention_options *options) {
+  return dispatch_paged_attention_loop_any<false>(out, query, key_cache, value_cache, block_tables,
+                                                  context_lens, scale, max_context_len, shape,
+                                                  options);
+}
+
+}  // namespace fa

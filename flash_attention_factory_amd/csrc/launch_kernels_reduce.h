@@ -1,0 +1,99 @@
+// Host launcher and dispatcher of the split-context path: the partition kernel
+// followed by the reduce kernel.
+//
+// Same role and argument list as upstream paged_attention_reduce/launch_kernels_reduce.h:
+// launch_paged_attn_v2 (:18-78) submits the attention kernel over
+// (sequences, kv heads, partitions) and then the reduce kernel over (sequences, heads),
+// returning both kernel times; dispatch_paged_attention (:80-197) picks the instance.
+// Upstream waits on the host between the two kernels (:56); here they are ordered by
+// the stream and nothing blocks unless timing is requested.
+#pragma once
+
+#include "launch_common.h"
+
+namespace fa {
+
+template <int HEAD_SIZE, typename QT, bool KV8>
+inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *key_cache,
+                                      const void *value_cache, const int32_t *block_tables,
+                                      const int32_t *context_lens, float scale,
+                                      int32_t /*max_context_len: validation only*/,
+                                      float *exp_sums, float *max_logits, float *tmp_out,
+                                      const fa_paged_attention_shape &shape, const Resolved &r) {
+  constexpr int NW = WavesPerGroup<true>::value;
+  const PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache,
+                                        value_cache, block_tables, context_lens, scale, shape, r);
+  KernelTimer timer(r.elapsed_us != nullptr, r.stream);
+  // kernel 1: one work-group per (kv head, partition, sequence); partitions past a
+  // sequence's length return at once and write nothing
+  // (paged_attention_kernel_v2.hpp:577-579 does the same)
+  const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+  FA_HIP_CHECK(timer.start(0));
+  hipLaunchKernelGGL((paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW>), grid, dim3(NW * 64), 0,
+                     r.stream, p);
+  FA_HIP_CHECK(hipGetLastError());
+  FA_HIP_CHECK(timer.stop(0));
+
+  // kernel 2: one wavefront per (head, sequence)
+  ReduceParams rp;
+  rp.out = out;
+  rp.exp_sums = exp_sums;
+  rp.max_logits = max_logits;
+  rp.tmp_out = tmp_out;
+  rp.context_lens = context_lens;
+  rp.num_heads = shape.num_heads;
+  rp.max_num_partitions = shape.max_num_partitions;
+  rp.partition_size = r.partition_size;
+  FA_HIP_CHECK(timer.start(1));
+  hipLaunchKernelGGL((paged_attn_reduce_kernel<HEAD_SIZE, QT>), dim3(shape.num_heads, shape.num_seqs),
+                     dim3(kReduceThreads), 0, r.stream, rp);
+  FA_HIP_CHECK(hipGetLastError());
+  FA_HIP_CHECK(timer.stop(1));
+  if (r.elapsed_us) {
+    FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
+    FA_HIP_CHECK(timer.read(1, &r.elapsed_us[1]));
+  }
+  return FA_OK;
+}
+
+template <bool KV8>
+inline fa_status dispatch_paged_attention_any(void *out, const void *query, const void *key_cache,
+                                              const void *value_cache,
+                                              const int32_t *block_tables,
+                                              const int32_t *context_lens, float scale,
+                                              int32_t max_context_len, float *exp_sums,
+                                              float *max_logits, float *tmp_out,
+                                              const fa_paged_attention_shape *shape,
+                                              const fa_paged_attention_options *options) {
+  Resolved r;
+  fa_status st = validate_and_resolve(out, query, key_cache, value_cache, block_tables, context_lens,
+                                      max_context_len, exp_sums, max_logits, tmp_out, shape, options,
+                                      KV8, /*split=*/true, &r);
+  if (st != FA_OK || r.validate_only) return st;
+  const bool bf16 = shape->q_dtype == FA_DTYPE_BF16;
+#define FA_V2_CASE(HS, QT)                                                                       \
+  return launch_paged_attn_v2<HS, QT, KV8>(out, query, key_cache, value_cache, block_tables,     \
+                                           context_lens, scale, max_context_len, exp_sums,       \
+                                           max_logits, tmp_out, *shape, r)
+  if (shape->head_size == 128) {
+    if (bf16) FA_V2_CASE(128, BF16);
+    FA_V2_CASE(128, F16);
+  }
+  if (bf16) FA_V2_CASE(64, BF16);
+  FA_V2_CASE(64, F16);
+#undef FA_V2_CASE
+}
+
+inline fa_status dispatch_paged_attention(void *out, const void *query, const void *key_cache,
+                                          const void *value_cache, const int32_t *block_tables,
+                                          const int32_t *context_lens, float scale,
+                                          int32_t max_context_len, float *exp_sums,
+                                          float *max_logits, float *tmp_out,
+                                          const fa_paged_attention_shape *shape,
+                                          const fa_paged_attention_options *options) {
+  return dispatch_paged_attention_any<false>(out, query, key_cache, value_cache, block_tables,
+                                             context_lens, scale, max_context_len, exp_sums,
+                                             max_logits, tmp_out, shape, options);
+}
+
+}  // namespace fa

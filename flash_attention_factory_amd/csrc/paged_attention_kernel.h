@@ -1,0 +1,374 @@
+// Paged-attention decode kernel for gfx950 (MI355X): the single-pass "loop" form
+// and the split-context "partition" form share this one template.
+//
+// Work decomposition (upstream: one work-group per (sequence, kv head[, partition]),
+// paged_attention_kernel_loop.hpp:602-607, paged_attention_kernel_v2.hpp:562-569;
+// the same here so K/V are read once per kv head):
+//   grid  = (num_kv_heads, partitions or 1, num_seqs)
+//   block = NW wavefronts; wavefront w takes the 32-token chunks w, w+NW, ... of the
+//           token range and keeps its own online-softmax state; states merge once at
+//           the end through LDS.  There is no barrier inside the streaming loop.
+//
+// Per chunk and wavefront (the query group's G <= 16 heads are the 16 MFMA columns):
+//   S^T[token, head] = K[token, :] . Q^T[:, head]      2 tiles x D/32 MFMA 16x16x32
+//   online softmax over tokens, fp32, base 2            VALU + two cross-row shuffles
+//   O^T[d, head]    += V^T[d, token] . P^T[token, head] D/16 MFMA 16x16x32
+// K rows enter the MFMA "A" operand exactly as they lie in HBM (lane 16r+i loads 16 B
+// of token i); V rows are loaded row-wise (16 lanes cover one token row) and
+// transposed inside each lane with byte permutes, so neither needs LDS.  The scores
+// come out of the first MFMA in the register layout the second MFMA wants for P^T.
+//
+// Arithmetic follows the upstream kernels (loop: paged_attention_kernel_loop.hpp:610-636,
+// split: paged_attention_kernel_v2.hpp:572-587, FP8: paged_attention_kernel_fp8_loop.hpp:
+// 328-333,540-545): fp32 scores scaled after the dot, tail tokens masked to -inf, sink
+// only in the first partition, probabilities rounded to the query dtype before P.V,
+// split form normalised inside the partition with (max, sum) written to scratch.
+#pragma once
+
+#include "paged_attention_policy.h"
+#include "paged_attention_utils.h"
+
+namespace fa {
+
+struct PagedAttnParams {
+  void *out;              // loop: [S,H,D] q dtype.  split: tmp_out [S,H,NP,D] fp32
+  float *exp_sums;        // split only: [S,H,NP]
+  float *max_logits;      // split only: [S,H,NP]
+  const void *query;      // [S,H,D]
+  const char *key_cache;
+  const char *value_cache;
+  const int32_t *block_tables;  // [S,MB]
+  const int32_t *context_lens;  // [S]
+  const void *sinks;            // [H] q dtype or nullptr
+  float score_scale_log2;       // sm_scale * fp8_scale * log2(e)
+  float out_scale;              // fp8_scale (1 for 16-bit caches)
+  int32_t num_heads;
+  int32_t group;                // query heads per kv head
+  int32_t max_blocks_per_seq;
+  int32_t max_num_partitions;
+  int32_t partition_size;       // tokens; multiple of 32
+  int32_t block_shift;          // log2(block_size)
+  int64_t kv_block_bytes;       // strides in BYTES
+  int64_t kv_token_bytes;
+  int64_t kv_head_bytes;
+};
+
+template <int D, bool KV8>
+struct KVChunk {
+  static constexpr int ROWB = D * (KV8 ? 1 : 2);  // bytes per token row
+  static constexpr int KL = ROWB / 64;            // 16-byte K loads per lane and tile
+  static constexpr int VW = ROWB / 64;            // dwords of V per lane and token
+  u32x4 k[2][KL];
+  uint32_t v[8][VW];
+};
+
+template <int D, typename QT, bool KV8, bool PART, int NW>
+__global__ void __launch_bounds__(NW * 64)
+paged_attn_kernel(const PagedAttnParams p) {
+  constexpr int ROWB = D * (KV8 ? 1 : 2);
+  constexpr int KL = ROWB / 64;
+  constexpr int KSTEPS = D / 32;   // MFMA k-steps across the head dimension
+  constexpr int NDT = D / 16;      // output d-tiles; lane row i of tile dt is d = i*NDT + dt
+  constexpr int VW = ROWB / 64;
+  constexpr int VB = VW * 4;       // bytes of V per lane and token
+  using Chunk = KVChunk<D, KV8>;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane >> 4;  // 16-lane row of the wavefront
+  const int i = lane & 15;  // position in the row: token (K), head (Q, P, O) or d-row (V)
+
+  const int kvh = blockIdx.x;
+  const int part = blockIdx.y;
+  const int seq = blockIdx.z;
+  const int G = p.group;
+
+  const int ctx = p.context_lens[seq];
+  const int tok_begin = PART ? part * p.partition_size : 0;
+  const int tok_end = PART ? min(ctx, tok_begin + p.partition_size) : ctx;
+  if (tok_begin >= tok_end) return;  // empty partition / empty sequence: nothing is written
+
+  const int c_begin = tok_begin / kChunkTokens;
+  const int c_end = (tok_end + kChunkTokens - 1) / kChunkTokens;
+  const int last_blk = (ctx - 1) >> p.block_shift;
+  const int blk_mask = (1 << p.block_shift) - 1;
+  const int32_t *table = p.block_tables + (int64_t)seq * p.max_blocks_per_seq;
+
+  // ---- Q^T as the MFMA "B" operand, one dword quad per k-step -------------------
+  // k-slot (r, e) of step c stands for head-dim element qd(c, r) + e; K uses the same map.
+  u32x4 qB[KSTEPS];
+  {
+    const int head = kvh * G + i;
+    const char *qrow = reinterpret_cast<const char *>(p.query) +
+                       ((int64_t)seq * p.num_heads + head) * (D * 2);
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c) {
+      const int d0 = KV8 ? ((c >> 1) * 4 + r) * 16 + (c & 1) * 8 : (c * 4 + r) * 8;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qB[c] = (i < G) ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
+    }
+  }
+
+  const char *kbase = p.key_cache + (int64_t)kvh * p.kv_head_bytes + r * 16;
+  const char *vbase = p.value_cache + (int64_t)kvh * p.kv_head_bytes + i * VB;
+
+  // ---- online softmax state, per lane ------------------------------------------------
+  // m: running max (base-2 units) of head i, identical in the four rows r.
+  // l: this lane's share of the running sum (its own tokens); rows are added at the end.
+  // acc[dt][e]: O^T[d = (4r+e)*NDT + dt][head i], un-normalised.
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (p.sinks != nullptr && wave == 0 && (!PART || part == 0) && i < G) {
+    // The sink is one more logit with a zero value row; it joins partition 0 only
+    // (paged_attention_kernel_loop.hpp:387-391, paged_attention_kernel_v2.hpp:373-376).
+    m = load_scalar16<QT>(reinterpret_cast<const char *>(p.sinks) + (kvh * G + i) * 2) * kLog2e;
+    l = (r == 0) ? 1.f : 0.f;
+  }
+
+  // Physical block ids of the two 16-token tiles of chunk ci (clamped so that a tile
+  // wholly past the context re-reads the last live block; it is masked below).
+  auto fetch_ids = [&](int ci, int &id0, int &id1) {
+    const int t0 = ci * kChunkTokens;
+    id0 = table[min(t0 >> p.block_shift, last_blk)];
+    id1 = table[min((t0 + kTileTokens) >> p.block_shift, last_blk)];
+  };
+
+  // Issue every global load of chunk ci into R.
+  auto issue = [&](Chunk &R, int ci, int id0, int id1) {
+    const int t0 = ci * kChunkTokens;
+    const int64_t off0 = (int64_t)id0 * p.kv_block_bytes +
+                         (int64_t)(t0 & blk_mask) * p.kv_token_bytes;
+    const int64_t off1 = (int64_t)id1 * p.kv_block_bytes +
+                         (int64_t)((t0 + kTileTokens) & blk_mask) * p.kv_token_bytes;
+    // K first (needed first), then V: waiting for K leaves the V loads in flight
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      const char *kp = kbase + (tile ? off1 : off0) + (int64_t)i * p.kv_token_bytes;
+#pragma unroll
+      for (int c = 0; c < KL; ++c) R.k[tile][c] = *reinterpret_cast<const u32x4 *>(kp + c * 64);
+    }
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      const char *vp = vbase + (tile ? off1 : off0) + (int64_t)(4 * r) * p.kv_token_bytes;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) VLoad<VW>::ld(R.v[tile * 4 + e], vp + e * p.kv_token_bytes);
+    }
+  };
+
+  // K "A" operand of k-step c for one tile: row i = token, 8 head-dim elements.
+  auto k_operand = [&](const Chunk &R, int tile, int c) -> u32x4 {
+    if constexpr (!KV8) {
+      return R.k[tile][c];
+    } else {
+      const u32x4 src = R.k[tile][c >> 1];
+      const int h = c & 1;
+      u32x4 o;
+      o[0] = e5m2_adjacent_pair<QT>(src[2 * h], 0);
+      o[1] = e5m2_adjacent_pair<QT>(src[2 * h], 1);
+      o[2] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 0);
+      o[3] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 1);
+      return o;
+    }
+  };
+
+  // V^T "A" operand of d-tile dt: row i = d-row, k-slots = this lane row's 8 tokens.
+  // In-lane transpose: R.v[e] holds token e's NDT consecutive head-dim elements.
+  auto v_operand = [&](const Chunk &R, int dt) -> u32x4 {
+    u32x4 o;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if constexpr (!KV8) {
+        const uint32_t y = R.v[2 * c][dt >> 1], x = R.v[2 * c + 1][dt >> 1];
+        o[c] = (dt & 1) ? ((y >> 16) | (x & 0xffff0000u)) : ((y & 0xffffu) | (x << 16));
+      } else {
+        const uint32_t y = (R.v[2 * c][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
+        const uint32_t x = (R.v[2 * c + 1][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
+        o[c] = e5m2_pair<QT>(y, x);
+      }
+    }
+    return o;
+  };
+
+  auto compute = [&](Chunk &R, int ci) {
+    // scores: S^T tile rows are tokens 4r+e of the tile, column i is the head
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c) {
+      s0 = mfma_16x16x32<QT>(k_operand(R, 0, c), qB[c], s0);
+      s1 = mfma_16x16x32<QT>(k_operand(R, 1, c), qB[c], s1);
+    }
+    float t[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      t[e] = s0[e] * p.score_scale_log2;
+      t[4 + e] = s1[e] * p.score_scale_log2;
+    }
+    const int t0 = ci * kChunkTokens;
+    if (t0 + kChunkTokens > tok_end) {  // wave-uniform: only the last chunk of the range
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int tok = t0 + (e >> 2) * kTileTokens + 4 * r + (e & 3);
+        if (tok >= tok_end) {
+          t[e] = -INFINITY;  // select, never multiply: the pool may hold NaN there
+#pragma unroll
+          for (int w = 0; w < VW; ++w) R.v[e][w] = 0u;
+        }
+      }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])),
+                     fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
+    mx = rows_max(mx);
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2(m - m_new);  // exp2(-inf) = 0 on the first chunk
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      t[e] = fast_exp2(t[e] - m_new);
+      ps += t[e];
+    }
+    l = l * alpha + ps;
+    m = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+    }
+    // P^T "B" operand: k-slots (r, e) = this lane's eight tokens, rounded to the q dtype
+    // (paged_attention_kernel_loop.hpp:404-407)
+    u32x4 pB;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) pB[c] = pack2<QT>(t[2 * c], t[2 * c + 1]);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) acc[dt] = mfma_16x16x32<QT>(v_operand(R, dt), pB, acc[dt]);
+  };
+
+  // ---- streaming loop: two register sets, loads of chunk n+1 in flight under chunk n --
+  // The last chunk is computed outside the issuing path so that no wait on the loads
+  // of the current chunk ever has to cover a path on which the next chunk was not issued.
+  {
+    Chunk A, B;
+    int ci = c_begin + wave;
+    if (ci < c_end) {
+      int id0, id1, nid0, nid1;
+      fetch_ids(ci, id0, id1);
+      issue(A, ci, id0, id1);
+      fetch_ids(ci + NW, nid0, nid1);
+      while (true) {
+        int cn = ci + NW;
+        if (cn >= c_end) {
+          compute(A, ci);
+          break;
+        }
+        issue(B, cn, nid0, nid1);
+        fetch_ids(cn + NW, nid0, nid1);
+        compute(A, ci);
+        ci = cn;
+        cn = ci + NW;
+        if (cn >= c_end) {
+          compute(B, ci);
+          break;
+        }
+        issue(A, cn, nid0, nid1);
+        fetch_ids(cn + NW, nid0, nid1);
+        compute(B, ci);
+        ci = cn;
+      }
+    }
+  }
+
+  l = rows_sum(l);
+
+  // ---- merge the NW wavefront states, normalise, store -------------------------------
+  constexpr int NR = NDT * 4;  // accumulator registers per lane
+  float M = m, L = l;
+  float o[NR];
+  int e_lo = 0;  // this wavefront stores rows e_lo .. e_lo + 4/NW - 1 of every d-tile
+  if constexpr (NW == 1) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e * NDT + dt] = acc[dt][e];
+  } else {
+    __shared__ float sm_m[NW][16];
+    __shared__ float sm_l[NW][16];
+    __shared__ float sm_acc[NW][NR][64];
+    if (r == 0) {
+      sm_m[wave][i] = m;
+      sm_l[wave][i] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sm_acc[wave][e * NDT + dt][lane] = acc[dt][e];
+    __syncthreads();
+    M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[w][i]);
+    float f[NW];
+    L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float mw = sm_m[w][i];
+      f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
+      L += f[w] * sm_l[w][i];
+    }
+    constexpr int EPW = 4 / NW;  // rows e per wavefront
+    static_assert(NW == 2 || NW == 4, "merge splits the 4 accumulator rows across wavefronts");
+    e_lo = wave * EPW;
+#pragma unroll
+    for (int idx = 0; idx < NR; ++idx) o[idx] = 0.f;
+#pragma unroll
+    for (int ee = 0; ee < EPW; ++ee)
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[w][(e_lo + ee) * NDT + dt][lane];
+        o[ee * NDT + dt] = a;  // compacted: slot ee <-> row e_lo + ee
+      }
+  }
+
+  if (i >= G) return;
+  const float inv = p.out_scale / L;
+  const int head = kvh * G + i;
+  const int n_e = (NW == 1) ? 4 : (4 / NW);
+  if constexpr (PART) {
+    const int64_t slot = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions + part;
+    float *dst = reinterpret_cast<float *>(p.out) + slot * D;
+#pragma unroll
+    for (int ee = 0; ee < n_e; ++ee) {
+      const int d0 = (4 * r + e_lo + ee) * NDT;
+#pragma unroll
+      for (int q4 = 0; q4 < NDT / 4; ++q4) {
+        f32x4 v = {o[ee * NDT + q4 * 4] * inv, o[ee * NDT + q4 * 4 + 1] * inv,
+                   o[ee * NDT + q4 * 4 + 2] * inv, o[ee * NDT + q4 * 4 + 3] * inv};
+        *reinterpret_cast<f32x4 *>(dst + d0 + q4 * 4) = v;
+      }
+    }
+    if (r == 0 && wave == 0) {
+      p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
+      p.exp_sums[slot] = L;
+    }
+  } else {
+    char *dst = reinterpret_cast<char *>(p.out) + ((int64_t)seq * p.num_heads + head) * (D * 2);
+#pragma unroll
+    for (int ee = 0; ee < n_e; ++ee) {
+      const int d0 = (4 * r + e_lo + ee) * NDT;
+      uint32_t w[NDT / 2];
+#pragma unroll
+      for (int q2 = 0; q2 < NDT / 2; ++q2)
+        w[q2] = pack2<QT>(o[ee * NDT + 2 * q2] * inv, o[ee * NDT + 2 * q2 + 1] * inv);
+      if constexpr (NDT == 8) {
+        u32x4 v = {w[0], w[1], w[2], w[3]};
+        *reinterpret_cast<u32x4 *>(dst + d0 * 2) = v;
+      } else {
+        u32x2 v = {w[0], w[1]};
+        *reinterpret_cast<u32x2 *>(dst + d0 * 2) = v;
+      }
+    }
+  }
+}
+
+}  // namespace fa

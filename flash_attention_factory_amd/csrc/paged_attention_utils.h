@@ -1,0 +1,156 @@
+// Wave-level helpers for the gfx950 paged-attention kernels: MFMA wrappers,
+// 16-bit packing, E5M2 dequantisation and cross-lane reductions.
+//
+// They take the place of the upstream helper header
+// (include/paged_attention_utils.hpp: padding_mask :314-363, mat_vec_mul_broadcast
+// :734-804, mat_vec_div_broadcast :806-879, group_reduce_t :881-960) but share no
+// structure with it: here a "tile" is the register image of a 16x16 MFMA operand in
+// one 64-lane wavefront.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+struct F16 {};   // query / output element tags
+struct BF16 {};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// D[16x16] += A[16x32] * B[32x16] on one wavefront.  Lane l = 16*r + i holds
+//   A[row i][k-slots 8r .. 8r+7]   (8 x 16 bit = 4 dwords)
+//   B[k-slots 8r .. 8r+7][col i]
+//   D[rows 4r .. 4r+3][col i]      (4 x fp32)
+// Which head-dim element or token a k-slot stands for is free as long as A and
+// B agree, which is what lets every operand be loaded straight from HBM.
+template <typename QT>
+__device__ __forceinline__ f32x4 mfma_16x16x32(u32x4 a, u32x4 b, f32x4 c);
+
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x32<F16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Two fp32 values -> one dword of two 16-bit floats (lo in bits 0..15), round to nearest even.
+template <typename QT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<F16>(float lo, float hi) {
+  f16x2 v = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename QT>
+__device__ __forceinline__ float load_scalar16(const void *p);
+template <>
+__device__ __forceinline__ float load_scalar16<F16>(const void *p) {
+  return (float)*reinterpret_cast<const _Float16 *>(p);
+}
+template <>
+__device__ __forceinline__ float load_scalar16<BF16>(const void *p) {
+  return (float)*reinterpret_cast<const __bf16 *>(p);
+}
+
+// E5M2 is binary16 cut to its top byte: byte b decodes to the fp16 with bits b << 8.
+// e5m2_pair<QT>(lo_byte, hi_byte) builds one dword holding the two decoded values in
+// the query dtype.  Bytes arrive already isolated in bits 0..7.
+template <typename QT>
+__device__ __forceinline__ uint32_t e5m2_pair(uint32_t lo_byte, uint32_t hi_byte);
+template <>
+__device__ __forceinline__ uint32_t e5m2_pair<F16>(uint32_t lo_byte, uint32_t hi_byte) {
+  return (lo_byte << 8) | (hi_byte << 24);
+}
+template <>
+__device__ __forceinline__ uint32_t e5m2_pair<BF16>(uint32_t lo_byte, uint32_t hi_byte) {
+  // v_cvt_scalef32_pk_bf16_bf8 decodes bytes 0 and 1 of its source; E5M2 -> bf16 is
+  // exact (2 mantissa bits, exponent range inside bf16's).
+  uint32_t two = lo_byte | (hi_byte << 8);
+  bf16x2 v = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(two, 1.0f, false);
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Dword w holds four E5M2 bytes; decode bytes (2*half, 2*half+1) to a 16-bit pair.
+template <typename QT>
+__device__ __forceinline__ uint32_t e5m2_adjacent_pair(uint32_t w, int half);
+template <>
+__device__ __forceinline__ uint32_t e5m2_adjacent_pair<F16>(uint32_t w, int half) {
+  return half == 0 ? (((w & 0xffu) << 8) | ((w & 0xff00u) << 16))
+                   : (((w >> 8) & 0xff00u) | (w & 0xff000000u));
+}
+template <>
+__device__ __forceinline__ uint32_t e5m2_adjacent_pair<BF16>(uint32_t w, int half) {
+  bf16x2 v = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, false)
+                       : __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, true);
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Reductions over the four 16-lane rows of a wavefront (lanes i, i+16, i+32, i+48).
+__device__ __forceinline__ float rows_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16));
+  v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Global loads of 4, 8 or 16 bytes per lane.
+template <int DWORDS>
+struct VLoad;
+template <>
+struct VLoad<4> {
+  static __device__ __forceinline__ void ld(uint32_t (&dst)[4], const char *p) {
+    u32x4 t = *reinterpret_cast<const u32x4 *>(p);
+    dst[0] = t[0]; dst[1] = t[1]; dst[2] = t[2]; dst[3] = t[3];
+  }
+};
+template <>
+struct VLoad<2> {
+  static __device__ __forceinline__ void ld(uint32_t (&dst)[2], const char *p) {
+    u32x2 t = *reinterpret_cast<const u32x2 *>(p);
+    dst[0] = t[0]; dst[1] = t[1];
+  }
+};
+template <>
+struct VLoad<1> {
+  static __device__ __forceinline__ void ld(uint32_t (&dst)[1], const char *p) {
+    dst[0] = *reinterpret_cast<const uint32_t *>(p);
+  }
+};
+
+}  // namespace fa

@@ -1,0 +1,103 @@
+"""Shared body of the four ``run`` functions: torch tensors -> C ABI call.
+
+Mirrors what the upstream pybind entry does with its arguments
+(paged_attention_loop/paged_attention_loop.cpp:44-79): pointers come from the tensors,
+sizes from their shapes -- num_seqs, num_heads, head_size from ``query``; num_kv_heads
+from ``key_cache.size(2)``; max_num_partitions from ``max_logits.size(2)``;
+max_blocks_per_seq from ``block_tables.size(1)``.  Unlike upstream, cache strides are
+read too, so a head-major pool passed as ``pool.permute(0, 2, 1, 3)`` works as well as
+the contiguous ``[blocks, block_size, kv_heads, head_size]`` tensor.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from .. import _cabi
+
+_scratch = {}
+
+
+def _fp32_scratch(tem_output: torch.Tensor, shape) -> torch.Tensor:
+    """Upstream keeps tem_output in the query dtype; the kernels here want fp32.  A
+    caller that passes a 16-bit tem_output gets a cached fp32 workspace instead."""
+    if tem_output.dtype == torch.float32 and tuple(tem_output.shape) == tuple(shape) \
+            and tem_output.is_contiguous():
+        return tem_output
+    key = (tem_output.device, tuple(shape))
+    buf = _scratch.get(key)
+    if buf is None:
+        _scratch.clear()
+        buf = torch.empty(shape, dtype=torch.float32, device=tem_output.device)
+        _scratch[key] = buf
+    return buf
+
+
+def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_output, output,
+             debug_output, query, key_cache, value_cache, block_tables, context_lens,
+             num_queries_per_tokens: int, sm_scale: float, fp8_scale: float, block_size: int,
+             max_context_len: int, alibi_slopes, sinks: Optional[torch.Tensor], softcap: float,
+             partition_size: int = 0, timed: bool = True) -> List[float]:
+    L = _cabi.load()
+    if not query.is_cuda:
+        raise RuntimeError("paged attention runs on the GPU only: `query` is not a device tensor")
+    for name, t in (("query", query), ("output", output), ("block_tables", block_tables),
+                    ("context_lens", context_lens)):
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    if query.dtype not in (torch.float16, torch.bfloat16) or output.dtype != query.dtype:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
+                                        "query/output must both be fp16 or both bf16")
+    if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
+                                        "block_tables and context_lens must be int32")
+    want_kv = (torch.float8_e5m2, torch.uint8) if fp8 else (query.dtype,)
+    if key_cache.dtype not in want_kv or value_cache.dtype != key_cache.dtype:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
+                                        f"key/value cache dtype {key_cache.dtype} not in {want_kv}")
+    if key_cache.dim() != 4 or key_cache.stride(3) != 1 or value_cache.stride() != key_cache.stride():
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
+                                        "caches must be 4-D [blocks, block_size, kv_heads, head_size] "
+                                        "views with a contiguous last dimension and equal strides")
+    S, H, D = query.shape
+    sh = _cabi.Shape()
+    sh.num_seqs, sh.num_heads, sh.head_size = S, H, D
+    sh.num_kv_heads = key_cache.size(2)
+    sh.block_size = block_size
+    sh.max_blocks_per_seq = block_tables.size(1)
+    sh.max_num_partitions = max_logits.size(2) if split else 1
+    sh.partition_size = partition_size
+    sh.kv_block_stride, sh.kv_token_stride, sh.kv_head_stride = (
+        key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
+    sh.q_dtype = _cabi.FA_DTYPE_BF16 if query.dtype == torch.bfloat16 else _cabi.FA_DTYPE_F16
+    if sh.num_kv_heads * num_queries_per_tokens != H:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_GROUP,
+                                        "Unsupported number of queries per token")
+    if key_cache.size(1) != block_size:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE,
+                                        "Unsupported head size or block size")
+    elapsed = (ctypes.c_float * 2)(0.0, 0.0)
+    op = _cabi.Options()
+    op.sinks = sinks.data_ptr() if sinks is not None else None
+    op.alibi_slopes = alibi_slopes.data_ptr() if alibi_slopes is not None else None
+    op.softcap = softcap
+    op.fp8_scale = fp8_scale
+    op.stream = torch.cuda.current_stream(query.device).cuda_stream
+    op.elapsed_us = ctypes.cast(elapsed, ctypes.POINTER(ctypes.c_float)) if timed else None
+    fn = getattr(L, entry)
+    args = [output.data_ptr(), query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
+            block_tables.data_ptr(), context_lens.data_ptr(), float(sm_scale), int(max_context_len)]
+    if split:
+        tmp = _fp32_scratch(tem_output, (S, H, sh.max_num_partitions, D))
+        if max_logits.dtype != torch.float32 or exp_sums.dtype != torch.float32 \
+                or not max_logits.is_contiguous() or not exp_sums.is_contiguous():
+            raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
+                                            "max_logits/exp_sums must be contiguous fp32")
+        args += [exp_sums.data_ptr(), max_logits.data_ptr(), tmp.data_ptr()]
+    with torch.cuda.device(query.device):
+        _cabi.check(fn(*args, ctypes.byref(sh), ctypes.byref(op)))
+    if not timed:
+        return []
+    return [elapsed[0], elapsed[1]] if split else [elapsed[0]]

@@ -1,0 +1,16 @@
+"""``paged_attention_fp8_loop.run``: the single-pass kernel over an FP8-E5M2 KV cache.
+
+Drop-in for the upstream extension module of the same name
+(paged_attention_fp8_loop/paged_attention_fp8_loop.cpp:21-39,84-86): same positional arguments, same return value
+(a list of kernel times in microseconds).
+"""
+from ._run import run_impl
+
+
+def run(max_logits, exp_sums, tem_output, output, debug_output, query, key_cache, value_cache,
+        block_tables, context_lens, num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
+        alibi_slopes, sinks, softcap):
+    return run_impl("fa_paged_attention_fp8_loop", False, True, max_logits, exp_sums, tem_output, output,
+                    debug_output, query, key_cache, value_cache, block_tables, context_lens,
+                    num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
+                    alibi_slopes, sinks, softcap)

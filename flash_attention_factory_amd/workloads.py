@@ -160,10 +160,19 @@ def _draw_lens(spec, S, gen):
     return lens.to(torch.int32)
 
 
+def _randn16_on(shape, device, seed, dtype):
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    return torch.randn(shape, generator=gen, device=device, dtype=torch.float16).to(dtype)
+
+
 def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs: Optional[int] = None,
-                pool_blocks: Optional[int] = None, device="cpu") -> Workload:
+                pool_blocks: Optional[int] = None, device="cpu", pools_on_device: bool = False) -> Workload:
     """One of the five measured configurations.  ``num_seqs``/``pool_blocks`` shrink
-    a configuration for CPU-sized parity runs without changing anything else."""
+    a configuration for CPU-sized parity runs without changing anything else.
+    ``pools_on_device`` draws the two KV pools with the target device's own generator
+    (same distribution, different bits) -- for throughput runs, where drawing a
+    gigabyte of normals on the host would dominate the run."""
     c = _CONFIGS[index]
     S = num_seqs or c["S"]
     H, Hk, D, B = c["H"], c["Hk"], c["D"], c["B"]
@@ -174,8 +183,12 @@ def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs
     query = _randn16((S, H, D), gen, qd)
     shape = (NB, Hk, B, D) if layout == HEAD_MAJOR else (NB, B, Hk, D)
     kv16 = torch.float16 if c["fp8"] else qd
-    k = _randn16(shape, gen, kv16)
-    v = _randn16(shape, gen, kv16)
+    if pools_on_device:
+        k = _randn16_on(shape, device, seed + 1, kv16)
+        v = _randn16_on(shape, device, seed + 2, kv16)
+    else:
+        k = _randn16(shape, gen, kv16)
+        v = _randn16(shape, gen, kv16)
     if c["fp8"]:
         # cast of fp16 N(0,1) samples, as test_paged_fp8cache.py:201-203 does
         k = k.to(torch.float8_e5m2)

@@ -1,0 +1,149 @@
+/*
+ * C ABI of the MI355X paged-attention decode library (libfa_paged_attention.so).
+ *
+ * Four entry points, one per upstream host launcher.  Each replaces the pybind11
+ * `run` function of one upstream extension module together with the dispatcher and
+ * launcher underneath it:
+ *
+ *   fa_paged_attention_loop        paged_attention_loop/paged_attention_loop.cpp:21-84
+ *                                  paged_attention_loop/launch_kernels_loop.h:16-173
+ *   fa_paged_attention_reduce      paged_attention_reduce/paged_attention_reduce.cpp:21-84
+ *                                  paged_attention_reduce/launch_kernels_reduce.h:18-197
+ *   fa_paged_attention_fp8_loop    paged_attention_fp8_loop/paged_attention_fp8_loop.cpp:21-86
+ *                                  paged_attention_fp8_loop/launch_kernels_fp8_loop.h:17-175
+ *   fa_paged_attention_fp8_reduce  paged_attention_fp8_reduce/paged_attention_fp8_reduce.cpp:21-86
+ *                                  paged_attention_fp8_reduce/launch_kernels_fp8_reduce.h:16-196
+ *
+ * All pointers except those in fa_paged_attention_options are DEVICE pointers owned
+ * by the caller for the duration of the call; nothing is retained.  No exception
+ * crosses this boundary: every function returns an fa_status and the text of the
+ * last failure on the calling thread is available from fa_last_error().
+ *
+ * Tensor shapes (row-major, innermost dimension contiguous):
+ *   out, query      [num_seqs, num_heads, head_size]            q_dtype (fp16 / bf16)
+ *   key_cache,      a pool of blocks addressed with explicit element strides
+ *   value_cache       element(block b, token t, kv head h, dim d) =
+ *                       base[b*kv_block_stride + t*kv_token_stride + h*kv_head_stride + d]
+ *                     16-bit caches hold q_dtype values, FP8 caches hold E5M2 bytes.
+ *                     upstream layout [blocks, block_size, kv_heads, head_size]
+ *                       -> strides (block_size*kv_heads*head_size, kv_heads*head_size, head_size)
+ *                     head-major layout [blocks, kv_heads, block_size, head_size]
+ *                       -> strides (kv_heads*block_size*head_size, head_size, block_size*head_size)
+ *   block_tables    [num_seqs, max_blocks_per_seq]              int32
+ *   context_lens    [num_seqs]                                  int32
+ *   exp_sums,       [num_seqs, num_heads, max_num_partitions]   fp32
+ *   max_logits
+ *   tmp_out         [num_seqs, num_heads, max_num_partitions, head_size]   fp32
+ *                   (the upstream keeps tmp_out in the query dtype,
+ *                    launch_kernels_reduce.h:20-21; fp32 drops one rounding step)
+ *
+ * Semantics follow the upstream kernels: query head h reads kv head
+ * h / (num_heads / num_kv_heads); tokens at or beyond context_lens[s] never
+ * contribute; an optional per-head sink logit joins the softmax denominator only;
+ * alibi_slopes and softcap are accepted and ignored exactly as upstream
+ * (paged_attention_kernel_loop.hpp:175-178,329-342 are commented out there).
+ * A sequence with context_lens[s] <= 0 leaves its rows of `out` untouched.
+ */
+#ifndef FA_PAGED_ATTENTION_H_
+#define FA_PAGED_ATTENTION_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fa_status {
+  FA_OK = 0,
+  FA_ERR_NULL_POINTER = 1,
+  /* upstream: std::runtime_error("Unsupported head size or block size"),
+   * launch_kernels_loop.h:170-172 */
+  FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE = 2,
+  /* upstream: std::runtime_error("Unsupported number of queries per token"),
+   * launch_kernels_loop.h:114-115 */
+  FA_ERR_UNSUPPORTED_GROUP = 3,
+  FA_ERR_UNSUPPORTED_DTYPE = 4,
+  FA_ERR_PARTITION_OVERFLOW = 5, /* max_context_len needs more than max_num_partitions */
+  FA_ERR_BAD_SHAPE = 6,          /* non-positive sizes, misaligned strides or pointers */
+  FA_ERR_RUNTIME = 7             /* a HIP call failed; see fa_last_error() */
+} fa_status;
+
+typedef enum fa_dtype { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 } fa_dtype;
+
+/* Shapes and strides that upstream reads off the torch tensors
+ * (paged_attention_loop.cpp:60-65) or fixes at compile time. */
+typedef struct fa_paged_attention_shape {
+  int32_t num_seqs;
+  int32_t num_heads;
+  int32_t num_kv_heads;
+  int32_t head_size;          /* 64 or 128 */
+  int32_t block_size;         /* power of two, >= 16 */
+  int32_t max_blocks_per_seq; /* row pitch of block_tables */
+  int32_t max_num_partitions; /* slots per (seq, head) in the scratch arrays; loop entries ignore it */
+  int32_t partition_size;     /* tokens per partition; 0 = upstream policy (512 for head 128,
+                                 256 for head 64, include/paged_attention_policy_v2.hpp:28,50) */
+  int64_t kv_block_stride;    /* in elements */
+  int64_t kv_token_stride;
+  int64_t kv_head_stride;
+  int32_t q_dtype;            /* fa_dtype of query, out, sinks and of a 16-bit cache */
+  int32_t reserved;
+} fa_paged_attention_shape;
+
+/* Everything upstream's `run` takes beyond the result-affecting list, plus stream
+ * and timing control.  A NULL options pointer means all defaults. */
+typedef struct fa_paged_attention_options {
+  const void *sinks;          /* device, [num_heads] in q_dtype, or NULL */
+  const float *alibi_slopes;  /* accepted, ignored */
+  float softcap;              /* accepted, ignored */
+  float fp8_scale;            /* FP8 entries only: K^ = dequant(K)*s, V^ = dequant(V)*s; 0 means 1.0 */
+  void *stream;               /* hipStream_t; NULL = the null stream */
+  float *elapsed_us;          /* HOST pointer or NULL.  Non-NULL: the call synchronises and writes
+                                 kernel times in microseconds, 1 float for loop entries,
+                                 2 floats (attention, reduce) for reduce entries -- what the
+                                 upstream `run` returns (launch_kernels_loop.h:53,
+                                 launch_kernels_reduce.h:76-77).  NULL: asynchronous, no timing. */
+  int32_t validate_only;      /* non-zero: check arguments, launch nothing */
+  int32_t reserved;
+} fa_paged_attention_options;
+
+/* Single-pass kernel: one launch, no scratch. */
+int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_cache,
+                                const void *value_cache, const int32_t *block_tables,
+                                const int32_t *context_lens, float scale, int32_t max_context_len,
+                                const fa_paged_attention_shape *shape,
+                                const fa_paged_attention_options *options);
+
+/* Split-context kernel followed by the reduce kernel. */
+int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
+                                  const void *value_cache, const int32_t *block_tables,
+                                  const int32_t *context_lens, float scale,
+                                  int32_t max_context_len, float *exp_sums, float *max_logits,
+                                  float *tmp_out, const fa_paged_attention_shape *shape,
+                                  const fa_paged_attention_options *options);
+
+/* FP8-E5M2 KV-cache variants: caches are bytes, dequantised in registers. */
+int32_t fa_paged_attention_fp8_loop(void *out, const void *query, const void *key_cache,
+                                    const void *value_cache, const int32_t *block_tables,
+                                    const int32_t *context_lens, float scale,
+                                    int32_t max_context_len,
+                                    const fa_paged_attention_shape *shape,
+                                    const fa_paged_attention_options *options);
+
+int32_t fa_paged_attention_fp8_reduce(void *out, const void *query, const void *key_cache,
+                                      const void *value_cache, const int32_t *block_tables,
+                                      const int32_t *context_lens, float scale,
+                                      int32_t max_context_len, float *exp_sums,
+                                      float *max_logits, float *tmp_out,
+                                      const fa_paged_attention_shape *shape,
+                                      const fa_paged_attention_options *options);
+
+/* Text of the last failure on the calling thread ("" if none). */
+const char *fa_last_error(void);
+
+/* ABI revision of this header. */
+int32_t fa_paged_attention_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_PAGED_ATTENTION_H_ */

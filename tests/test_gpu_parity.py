@@ -1,0 +1,164 @@
+"""Parity of the HIP kernels (through lib.paged_attention_*.run -> C ABI) with the CPU
+oracle on the same seeded inputs.  Tolerance: atol = rtol = 1e-2 on fp16/bf16 outputs,
+as the benchmark contract states; the upstream relative rule
+(err <= 3 * err_of_a_16-bit-torch-evaluation + 1e-5, test_paged.py:603-604) is checked
+in the form err <= 3 * err(oracle kernel model) + 1e-5 where the kernel model rounds
+where the upstream kernels round."""
+import math
+
+import pytest
+import torch
+
+from flash_attention_factory_amd import workloads as W
+from _torch_ref import call_oracle
+
+pytestmark = pytest.mark.gpu
+
+ATOL = RTOL = 1e-2
+
+
+def _dev():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch.device("cuda:0")
+
+
+def _run(w_cpu, kernel, **kw):
+    from flash_attention_factory_amd import runner
+    w = w_cpu.to(_dev())
+    bufs = runner.alloc_buffers(w, **kw)
+    times = runner.run_workload(w, kernel, bufs)
+    torch.cuda.synchronize()
+    return bufs, times
+
+
+def _check(out, w_cpu, oracle, label):
+    ref16, ref32 = call_oracle(oracle.attention_ref, w_cpu, want_f32=True)
+    got = out.float().cpu()
+    err = (got - ref32).abs().max().item()
+    mag = ref32.abs().max().item()
+    print(f"{label}: max|out-ref| = {err:.3e}, max|ref| = {mag:.3e}, rel = {err / mag:.3e}", flush=True)
+    assert torch.isfinite(got).all(), label
+    torch.testing.assert_close(got, ref32, atol=ATOL, rtol=RTOL, msg=lambda m: f"{label}: {m}")
+    # upstream-style relative gate against the rounding-faithful kernel model
+    _, model32 = call_oracle(oracle.kernel_loop, w_cpu, partition_size=w_cpu.partition_size, want_f32=True)
+    ulp = 2.0 ** (-8 if w_cpu.query.dtype == torch.bfloat16 else -11) * mag
+    bar = 3 * max((model32 - ref32).abs().max().item(), ulp) + 1e-5
+    assert err <= bar, f"{label}: err {err:.3e} above relative bar {bar:.3e}"
+
+
+SMALL = {  # measured configurations cut down so the oracle finishes in seconds
+    0: dict(),
+    1: dict(num_seqs=4, pool_blocks=512),
+    2: dict(num_seqs=1, pool_blocks=2048),
+    3: dict(num_seqs=4, pool_blocks=512),
+    4: dict(num_seqs=6, pool_blocks=8192),
+}
+
+
+@pytest.mark.parametrize("index", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("layout", [W.HEAD_MAJOR, W.TOKEN_MAJOR])
+def test_measured_configs(oracle, index, layout):
+    w = W.make_config(index, layout=layout, **SMALL[index])
+    kernel = W.CONFIG_KERNEL[index]
+    bufs, times = _run(w, kernel)
+    assert len(times) == (2 if "reduce" in kernel else 1) and all(t > 0 for t in times)
+    _check(bufs.out, w, oracle, f"{w.name}/{layout}")
+
+
+@pytest.mark.parametrize("index", [0, 1, 3])
+def test_other_kernel_on_same_config(oracle, index):
+    """Every configuration also runs through the other kernel of its cache type."""
+    w = W.make_config(index, **SMALL[index])
+    kernel = {"loop": "reduce", "fp8_loop": "fp8_reduce"}[W.CONFIG_KERNEL[index]]
+    bufs, _ = _run(w, kernel)
+    _check(bufs.out, w, oracle, f"{w.name} via {kernel}")
+
+
+GRID = [  # a slice of the upstream grid (test_paged.py:211-256): groups 8,8,5,7,6,4,3,2,1
+    dict(batch_size=2, nheads=8, nheads_k=1, d=128, seqlen_k=339, varlen=True, has_sinks=True),
+    dict(batch_size=1, nheads=16, nheads_k=2, d=64, seqlen_k=1024, varlen=False, has_sinks=False),
+    dict(batch_size=2, nheads=10, nheads_k=2, d=128, seqlen_k=800, varlen=True, has_sinks=False),
+    dict(batch_size=2, nheads=14, nheads_k=2, d=64, seqlen_k=799, varlen=True, has_sinks=True),
+    dict(batch_size=1, nheads=12, nheads_k=2, d=128, seqlen_k=2048, varlen=False, has_sinks=True),
+    dict(batch_size=2, nheads=8, nheads_k=2, d=64, seqlen_k=128, varlen=True, has_sinks=False),
+    dict(batch_size=2, nheads=6, nheads_k=2, d=128, seqlen_k=256, varlen=False, has_sinks=True),
+    dict(batch_size=1, nheads=4, nheads_k=2, d=64, seqlen_k=20000, varlen=True, has_sinks=False),
+    dict(batch_size=2, nheads=2, nheads_k=2, d=128, seqlen_k=2048, varlen=True, has_sinks=True),
+]
+
+
+@pytest.mark.parametrize("case", GRID, ids=lambda c: "h{nheads}x{nheads_k}_d{d}_s{seqlen_k}".format(**c))
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("split", [False, True])
+def test_upstream_grid_slice(oracle, case, fp8, split):
+    w = W.make_test_shaped(fp8=fp8, **case)
+    kernel = ("fp8_" if fp8 else "") + ("reduce" if split else "loop")
+    bufs, _ = _run(w, kernel)
+    _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_partition_scratch_matches_kernel_model(oracle, fp8):
+    """exp_sums / max_logits / tmp_out against the restated upstream arithmetic; slots of
+    partitions past a sequence's length stay untouched (paged_attention_kernel_v2.hpp:577-579)."""
+    w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=1300, varlen=True,
+                           has_sinks=True, fp8=fp8, seed=7)
+    w.context_lens = torch.tensor([1300, 700], dtype=torch.int32)
+    NP = 5  # one slot more than any sequence needs
+    bufs, _ = _run(w, "fp8_reduce" if fp8 else "reduce", max_num_partitions=NP)
+    es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=w.partition_size,
+                              max_num_partitions=NP)
+    g_es, g_ml, g_tmp = bufs.exp_sums.cpu(), bufs.max_logits.cpu(), bufs.tmp_out.cpu()
+    for s in range(2):
+        live = math.ceil(int(w.context_lens[s]) / w.partition_size)
+        torch.testing.assert_close(g_ml[s, :, :live], ml[s, :, :live], atol=1e-4, rtol=1e-5)
+        torch.testing.assert_close(g_es[s, :, :live], es[s, :, :live], atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(g_tmp[s, :, :live], tmp[s, :, :live], atol=2e-3, rtol=1e-2)
+        assert torch.isnan(g_ml[s, :, live:]).all() and torch.isnan(g_tmp[s, :, live:]).all()
+
+
+def test_edge_cases(oracle):
+    # context lengths 1, 15, 16, 17, 31, 32, 33 and one exactly on a partition boundary
+    w = W.make_config(0, num_seqs=8, pool_blocks=256)
+    lens = torch.tensor([1, 15, 16, 17, 31, 32, 33, 256], dtype=torch.int32)
+    w.context_lens = lens
+    for kernel in ("loop", "reduce"):
+        bufs, _ = _run(w, kernel)
+        _check(bufs.out, w, oracle, f"edge lens/{kernel}")
+    # rows past context_len hold NaN: they must not leak (select, not multiply)
+    w2 = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=300, varlen=True,
+                            has_sinks=False, seed=11)
+    base_k, base_v = w2.key_cache.clone(), w2.value_cache.clone()
+    for s in range(2):
+        n = int(w2.context_lens[s])
+        for t in range(n, w2.block_tables.shape[1] * w2.block_size):
+            blk = int(w2.block_tables[s, t // w2.block_size])
+            w2.key_cache[blk, t % w2.block_size] = float("nan")
+            w2.value_cache[blk, t % w2.block_size] = float("nan")
+    for kernel in ("loop", "reduce"):
+        bufs, _ = _run(w2, kernel)
+        w2.key_cache, w2.value_cache = base_k, base_v
+        _check(bufs.out, w2, oracle, f"nan tail/{kernel}")
+        w2.key_cache, w2.value_cache = w2.key_cache.clone(), w2.value_cache.clone()
+    # a zero-length sequence leaves its output rows untouched
+    w3 = W.make_config(0)
+    w3.context_lens = torch.tensor([0, 40, 0, 7], dtype=torch.int32)
+    bufs, _ = _run(w3, "loop")
+    out = bufs.out.cpu()
+    assert (out[0] == 0).all() and (out[2] == 0).all()
+    ref = call_oracle(oracle.attention_ref, w3)
+    torch.testing.assert_close(out[[1, 3]].float(), ref[[1, 3]].float(), atol=ATOL, rtol=RTOL)
+
+
+def test_bf16_and_fp8_scale(oracle):
+    # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
+    w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,
+                           has_sinks=True, dtype=torch.bfloat16)
+    bufs, _ = _run(w, "loop")
+    _check(bufs.out, w, oracle, "bf16 cache/loop")
+    w8 = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=64, seqlen_k=700, varlen=True,
+                            has_sinks=False, dtype=torch.bfloat16, fp8=True)
+    w8.fp8_scale = 0.5  # parity unpinned upstream (tests only pass 1.0); checked against our reading
+    for kernel in ("fp8_loop", "fp8_reduce"):
+        bufs, _ = _run(w8, kernel)
+        _check(bufs.out, w8, oracle, f"bf16 q, fp8 cache, scale 0.5/{kernel}")
