@@ -46,7 +46,7 @@ class Shape(ctypes.Structure):
         ("kv_token_stride", ctypes.c_int64),
         ("kv_head_stride", ctypes.c_int64),
         ("q_dtype", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("num_pool_blocks", ctypes.c_int32),
     ]
 
 

@@ -81,6 +81,7 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
                 "%d a power of two >= 16)", s->head_size, s->block_size);
   if (s->num_seqs <= 0 || s->num_heads <= 0 || s->num_kv_heads <= 0 || s->max_blocks_per_seq <= 0)
     return fail(FA_ERR_BAD_SHAPE, "num_seqs, num_heads, num_kv_heads and max_blocks_per_seq must be positive");
+  if (s->num_pool_blocks < 0) return fail(FA_ERR_BAD_SHAPE, "num_pool_blocks must be >= 0");
   if (s->num_seqs > 65535)
     return fail(FA_ERR_BAD_SHAPE, "num_seqs %d exceeds the grid limit 65535", s->num_seqs);
   if (s->num_heads % s->num_kv_heads != 0)
@@ -147,6 +148,7 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.max_num_partitions = s.max_num_partitions;
   p.partition_size = r.partition_size;
   p.block_shift = ilog2(s.block_size);
+  p.max_block_id = s.num_pool_blocks > 0 ? s.num_pool_blocks - 1 : INT32_MAX;
   p.kv_block_bytes = s.kv_block_stride * r.kv_elem_bytes;
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;

@@ -9,6 +9,8 @@
 // the stream and nothing blocks unless timing is requested.
 #pragma once
 
+#include <algorithm>
+
 #include "launch_common.h"
 
 namespace fa {
@@ -44,6 +46,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   rp.num_heads = shape.num_heads;
   rp.max_num_partitions = shape.max_num_partitions;
   rp.partition_size = r.partition_size;
+  rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
   FA_HIP_CHECK(timer.start(1));
   hipLaunchKernelGGL((paged_attn_reduce_kernel<HEAD_SIZE, QT>), dim3(shape.num_heads, shape.num_seqs),
                      dim3(kReduceThreads), 0, r.stream, rp);

@@ -48,6 +48,7 @@ struct PagedAttnParams {
   int32_t max_num_partitions;
   int32_t partition_size;       // tokens; multiple of 32
   int32_t block_shift;          // log2(block_size)
+  int32_t max_block_id;         // block ids are clamped into [0, max_block_id]
   int64_t kv_block_bytes;       // strides in BYTES
   int64_t kv_token_bytes;
   int64_t kv_head_bytes;
@@ -83,7 +84,8 @@ paged_attn_kernel(const PagedAttnParams p) {
   const int seq = blockIdx.z;
   const int G = p.group;
 
-  const int ctx = p.context_lens[seq];
+  // a length the block table cannot hold is cut to what it holds
+  const int ctx = min(p.context_lens[seq], p.max_blocks_per_seq << p.block_shift);
   const int tok_begin = PART ? part * p.partition_size : 0;
   const int tok_end = PART ? min(ctx, tok_begin + p.partition_size) : ctx;
   if (tok_begin >= tok_end) return;  // empty partition / empty sequence: nothing is written
@@ -132,8 +134,9 @@ paged_attn_kernel(const PagedAttnParams p) {
   // wholly past the context re-reads the last live block; it is masked below).
   auto fetch_ids = [&](int ci, int &id0, int &id1) {
     const int t0 = ci * kChunkTokens;
-    id0 = table[min(t0 >> p.block_shift, last_blk)];
-    id1 = table[min((t0 + kTileTokens) >> p.block_shift, last_blk)];
+    id0 = min((uint32_t)table[min(t0 >> p.block_shift, last_blk)], (uint32_t)p.max_block_id);
+    id1 = min((uint32_t)table[min((t0 + kTileTokens) >> p.block_shift, last_blk)],
+              (uint32_t)p.max_block_id);
   };
 
   // Issue every global load of chunk ci into R.

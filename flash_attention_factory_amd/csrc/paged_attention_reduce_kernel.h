@@ -24,6 +24,7 @@ struct ReduceParams {
   int32_t num_heads;
   int32_t max_num_partitions;
   int32_t partition_size;
+  int32_t max_context;  // max_blocks_per_seq * block_size: lengths are cut to it
 };
 
 template <int D, typename QT>
@@ -32,7 +33,7 @@ __global__ void __launch_bounds__(64) paged_attn_reduce_kernel(const ReduceParam
   const int lane = threadIdx.x;
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
-  const int ctx = p.context_lens[seq];
+  const int ctx = min(p.context_lens[seq], p.max_context);
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;
   np = min(np, p.max_num_partitions);

@@ -71,6 +71,7 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     sh.partition_size = partition_size
     sh.kv_block_stride, sh.kv_token_stride, sh.kv_head_stride = (
         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
+    sh.num_pool_blocks = key_cache.size(0)
     sh.q_dtype = _cabi.FA_DTYPE_BF16 if query.dtype == torch.bfloat16 else _cabi.FA_DTYPE_F16
     if sh.num_kv_heads * num_queries_per_tokens != H:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_GROUP,

@@ -167,12 +167,14 @@ def _randn16_on(shape, device, seed, dtype):
 
 
 def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs: Optional[int] = None,
-                pool_blocks: Optional[int] = None, device="cpu", pools_on_device: bool = False) -> Workload:
+                pool_blocks: Optional[int] = None, device="cpu", pools_on_device: bool = False,
+                lens=None) -> Workload:
     """One of the five measured configurations.  ``num_seqs``/``pool_blocks`` shrink
     a configuration for CPU-sized parity runs without changing anything else.
     ``pools_on_device`` draws the two KV pools with the target device's own generator
     (same distribution, different bits) -- for throughput runs, where drawing a
-    gigabyte of normals on the host would dominate the run."""
+    gigabyte of normals on the host would dominate the run.  ``lens`` replaces the
+    drawn context lengths (the block tables are dealt for the lengths in force)."""
     c = _CONFIGS[index]
     S = num_seqs or c["S"]
     H, Hk, D, B = c["H"], c["Hk"], c["D"], c["B"]
@@ -194,7 +196,9 @@ def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs
         k = k.to(torch.float8_e5m2)
         v = v.to(torch.float8_e5m2)
     perm = torch.randperm(NB, generator=gen, dtype=torch.int64).to(torch.int32)
-    lens = _draw_lens(c["lens"], S, gen)
+    drawn = _draw_lens(c["lens"], S, gen)
+    lens = drawn if lens is None else torch.as_tensor(lens, dtype=torch.int32)
+    assert lens.numel() == S
     tables = _deal_block_tables(lens, B, perm)
     w = Workload(
         name=config_names()[index], query=query, key_cache=k, value_cache=v, block_tables=tables,

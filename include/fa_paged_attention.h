@@ -42,7 +42,9 @@
  * contribute; an optional per-head sink logit joins the softmax denominator only;
  * alibi_slopes and softcap are accepted and ignored exactly as upstream
  * (paged_attention_kernel_loop.hpp:175-178,329-342 are commented out there).
- * A sequence with context_lens[s] <= 0 leaves its rows of `out` untouched.
+ * A sequence with context_lens[s] <= 0 leaves its rows of `out` untouched; a
+ * context length above max_blocks_per_seq * block_size is cut to that bound, so the
+ * kernels never read past a row of block_tables.
  */
 #ifndef FA_PAGED_ATTENTION_H_
 #define FA_PAGED_ATTENTION_H_
@@ -86,7 +88,10 @@ typedef struct fa_paged_attention_shape {
   int64_t kv_token_stride;
   int64_t kv_head_stride;
   int32_t q_dtype;            /* fa_dtype of query, out, sinks and of a 16-bit cache */
-  int32_t reserved;
+  int32_t num_pool_blocks;    /* blocks in each cache pool, or 0 if unknown.  When given, block ids
+                                 read from block_tables are clamped into [0, num_pool_blocks) so a
+                                 corrupt table cannot make the kernel touch memory outside the pool
+                                 (upstream has no such guard) */
 } fa_paged_attention_shape;
 
 /* Everything upstream's `run` takes beyond the result-affecting list, plus stream

@@ -119,9 +119,7 @@ def test_partition_scratch_matches_kernel_model(oracle, fp8):
 
 def test_edge_cases(oracle):
     # context lengths 1, 15, 16, 17, 31, 32, 33 and one exactly on a partition boundary
-    w = W.make_config(0, num_seqs=8, pool_blocks=256)
-    lens = torch.tensor([1, 15, 16, 17, 31, 32, 33, 256], dtype=torch.int32)
-    w.context_lens = lens
+    w = W.make_config(0, num_seqs=8, pool_blocks=256, lens=[1, 15, 16, 17, 31, 32, 33, 256])
     for kernel in ("loop", "reduce"):
         bufs, _ = _run(w, kernel)
         _check(bufs.out, w, oracle, f"edge lens/{kernel}")
@@ -141,8 +139,7 @@ def test_edge_cases(oracle):
         _check(bufs.out, w2, oracle, f"nan tail/{kernel}")
         w2.key_cache, w2.value_cache = w2.key_cache.clone(), w2.value_cache.clone()
     # a zero-length sequence leaves its output rows untouched
-    w3 = W.make_config(0)
-    w3.context_lens = torch.tensor([0, 40, 0, 7], dtype=torch.int32)
+    w3 = W.make_config(0, lens=[0, 40, 0, 7])
     bufs, _ = _run(w3, "loop")
     out = bufs.out.cpu()
     assert (out[0] == 0).all() and (out[2] == 0).all()
