@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Throughput of the paged-attention decode path on one MI355X.
+
+A "step" is one call of the hot path (`lib.paged_attention_loop.run`) over the
+Llama-2-7B-shaped decode batch (configuration 1: 32 sequences, 32 heads, head size
+128, block size 16, context lengths uniform in [512, 2048], fp16).  KV pools are
+resident in HBM before timing starts; three pool clones are rotated so that no call
+finds its blocks in the 256 MB Infinity Cache (the upstream perf loop rotates 50
+clones for the same reason, test_paged.py:488-496).
+
+value        algorithmic bytes per step / wall time per step over K asynchronous steps
+roofline     per-kernel HIP-event time on the launch stream (the library's own
+             elapsed_us path), HBM-bound
+cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTorch
+             reference) on the same workload on this box's host cores
+configs      the other four configurations, each timed the same way
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# (summaries under profiles/); None where not yet measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def _clones(w, torch):
+    pool_bytes = w.key_cache.numel() * w.key_cache.element_size()
+    n = max(2, min(8, math.ceil((1 << 30) / pool_bytes) + 1))
+    ks = [w.key_cache] + [w.key_cache.clone() for _ in range(n - 1)]
+    vs = [w.value_cache] + [w.value_cache.clone() for _ in range(n - 1)]
+    return ks, vs
+
+
+def _time_config(index, steps, warmup, torch, W, runner, dev):
+    w = W.make_config(index, device=dev, pools_on_device=True)
+    kernel = W.CONFIG_KERNEL[index]
+    ks, vs = _clones(w, torch)
+    bufs = runner.alloc_buffers(w)
+    n = len(ks)
+    for it in range(warmup):
+        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for it in range(steps):
+        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    # per-kernel durations from HIP events on the launch stream
+    ev = []
+    for it in range(steps):
+        ev.append(runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n]))
+    ev_t = torch.tensor(ev, dtype=torch.float64)
+    res = dict(
+        workload=w.name, kernel=kernel, steps=steps,
+        ms_per_step=wall / steps * 1e3,
+        algorithmic_bytes=w.algorithmic_bytes(),
+        scratch_bytes=w.scratch_bytes() if "reduce" in kernel else 0,
+        kernel_us_mean=[float(x) for x in ev_t.mean(0)],
+        kernel_us_median=[float(x) for x in ev_t.median(0).values],
+        us_per_call=float(ev_t.sum(1).mean()),
+        pool_clones=n,
+    )
+    res["gbps_wall"] = res["algorithmic_bytes"] / (wall / steps) / 1e9
+    res["gbps_kernels"] = res["algorithmic_bytes"] / (res["us_per_call"] * 1e-6) / 1e9
+    res["hbm_frac"] = res["gbps_kernels"] / HBM_PEAK_GBPS
+    # the dominant kernel alone (the attention kernel; the reduce kernel is reported beside it)
+    res["gbps_attention_kernel"] = res["algorithmic_bytes"] / (res["kernel_us_mean"][0] * 1e-6) / 1e9
+    return w, res
+
+
+def _cpu_baseline(index, torch, W, budget_s=12.0):
+    from oracle import oracle as O
+    w = W.make_config(index)  # CPU generator, seeded
+    def call():
+        return O.attention_ref(w.query, w.key_cache, w.value_cache, w.block_tables, w.context_lens,
+                               scale=w.scale, block_size=w.block_size, kv_strides=w.kv_strides(),
+                               num_kv_heads=w.num_kv_heads, sinks=w.sinks, fp8_scale=w.fp8_scale)
+    call()  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        call()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or reps >= 200:
+            break
+    per = dt / reps
+    return dict(value=w.algorithmic_bytes() / per / 1e9, unit="GB/s", cores=O.num_threads(), kind="port",
+                ms_per_call=per * 1e3,
+                sample=f"full {w.name} workload (seed 0), {reps} repetitions of the C/OpenMP oracle "
+                       f"oracle_attention_ref, {dt:.1f} s")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--configs", type=str, default="0,2,3,4",
+                    help="other configurations to time besides configuration 1 ('' for none)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this path has no multi-GPU form in this build "
+              f"(--gpus {args.gpus} refused)", file=sys.stderr)
+        return 2
+
+    import torch
+    from flash_attention_factory_amd import _cabi, runner, workloads as W
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    _cabi.load()  # raises if the HIP library was not built: there is no fallback
+    dev = torch.device("cuda:0")
+
+    w, main_res = _time_config(1, args.steps, args.warmup, torch, W, runner, dev)
+    others = []
+    for idx in [int(x) for x in args.configs.split(",") if x.strip() != ""]:
+        del w
+        torch.cuda.empty_cache()
+        w, r = _time_config(idx, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+        others.append(r)
+
+    kernel_us = main_res["kernel_us_mean"][0]
+    achieved = main_res["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9
+    line = {
+        "metric": "achieved HBM GB/s, fp16 paged decode (loop kernel)",
+        "value": main_res["gbps_wall"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16",
+        "data": "synthetic",
+        "config": {"workload": "config1: fp16 loop kernel, S32 H32 Hk32 D128 B16 ctx U[512,2048], "
+                               "4096-block head-major pool, shuffled block tables",
+                   "us_per_call": main_res["us_per_call"],
+                   "algorithmic_bytes": main_res["algorithmic_bytes"],
+                   "hbm_frac_of_8TBps": main_res["hbm_frac"]},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("config1_loop"),
+                     "kernel": "paged_attn_kernel<128, F16, kv16, loop, 4 waves>",
+                     "kernel_us": kernel_us},
+        "configs": others,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = _cpu_baseline(1, torch, W)
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

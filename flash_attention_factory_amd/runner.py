@@ -50,7 +50,7 @@ def alloc_buffers(w: Workload, max_num_partitions: Optional[int] = None, fill: f
 
 def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
                  key_cache: Optional[torch.Tensor] = None,
-                 value_cache: Optional[torch.Tensor] = None) -> List[float]:
+                 value_cache: Optional[torch.Tensor] = None, timed: bool = True) -> List[float]:
     """One call of ``lib.paged_attention_<kernel>.run``; returns its kernel times (us).
     ``key_cache``/``value_cache`` substitute pool clones of the same layout."""
     if kernel.startswith("fp8") != w.is_fp8:
@@ -65,5 +65,5 @@ def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
             w.block_tables, w.context_lens, G, w.scale)
     tail = (w.block_size, max_ctx, bufs.alibi, w.sinks, -1.0)
     if w.is_fp8:
-        return mod.run(*head, w.fp8_scale, *tail)
-    return mod.run(*head, *tail)
+        return mod.run(*head, w.fp8_scale, *tail, timed=timed)
+    return mod.run(*head, *tail, timed=timed)
