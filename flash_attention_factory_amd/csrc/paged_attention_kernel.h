@@ -284,10 +284,14 @@ paged_attn_kernel(const PagedAttnParams p) {
   l = rows_sum(l);
 
   // ---- merge the NW wavefront states, normalise, store -------------------------------
-  constexpr int NR = NDT * 4;  // accumulator registers per lane
+  // A lane's NR accumulator values are NR consecutive head-dim elements of head i:
+  // d = 4r*NDT + idx with idx = e*NDT + dt.  After the merge wavefront w owns the slice
+  // idx in [w*SL, (w+1)*SL) of every lane and stores it.
+  constexpr int NR = NDT * 4;
+  constexpr int SL = NR / NW;
+  static_assert(NR % NW == 0 && SL >= 2, "output slice per wavefront must hold >= 2 elements");
   float M = m, L = l;
-  float o[NR];
-  int e_lo = 0;  // this wavefront stores rows e_lo .. e_lo + 4/NW - 1 of every d-tile
+  float o[SL];
   if constexpr (NW == 1) {
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
@@ -317,59 +321,57 @@ paged_attn_kernel(const PagedAttnParams p) {
       f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
       L += f[w] * sm_l[w][i];
     }
-    constexpr int EPW = 4 / NW;  // rows e per wavefront
-    static_assert(NW == 2 || NW == 4, "merge splits the 4 accumulator rows across wavefronts");
-    e_lo = wave * EPW;
 #pragma unroll
-    for (int idx = 0; idx < NR; ++idx) o[idx] = 0.f;
+    for (int k = 0; k < SL; ++k) {
+      float a = 0.f;
 #pragma unroll
-    for (int ee = 0; ee < EPW; ++ee)
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        float a = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[w][(e_lo + ee) * NDT + dt][lane];
-        o[ee * NDT + dt] = a;  // compacted: slot ee <-> row e_lo + ee
-      }
+      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[w][wave * SL + k][lane];
+      o[k] = a;
+    }
   }
 
   if (i >= G) return;
   const float inv = p.out_scale / L;
   const int head = kvh * G + i;
-  const int n_e = (NW == 1) ? 4 : (4 / NW);
+  const int d0 = 4 * r * NDT + wave * SL;  // first head-dim element this lane stores (wave = 0 if NW == 1)
   if constexpr (PART) {
     const int64_t slot = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions + part;
-    float *dst = reinterpret_cast<float *>(p.out) + slot * D;
+    float *dst = reinterpret_cast<float *>(p.out) + slot * D + d0;
+    if constexpr (SL % 4 == 0) {
 #pragma unroll
-    for (int ee = 0; ee < n_e; ++ee) {
-      const int d0 = (4 * r + e_lo + ee) * NDT;
-#pragma unroll
-      for (int q4 = 0; q4 < NDT / 4; ++q4) {
-        f32x4 v = {o[ee * NDT + q4 * 4] * inv, o[ee * NDT + q4 * 4 + 1] * inv,
-                   o[ee * NDT + q4 * 4 + 2] * inv, o[ee * NDT + q4 * 4 + 3] * inv};
-        *reinterpret_cast<f32x4 *>(dst + d0 + q4 * 4) = v;
+      for (int k = 0; k < SL; k += 4) {
+        f32x4 v = {o[k] * inv, o[k + 1] * inv, o[k + 2] * inv, o[k + 3] * inv};
+        *reinterpret_cast<f32x4 *>(dst + k) = v;
       }
+    } else {
+#pragma unroll
+      for (int k = 0; k < SL; ++k) dst[k] = o[k] * inv;
     }
     if (r == 0 && wave == 0) {
       p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
       p.exp_sums[slot] = L;
     }
   } else {
-    char *dst = reinterpret_cast<char *>(p.out) + ((int64_t)seq * p.num_heads + head) * (D * 2);
+    char *dst = reinterpret_cast<char *>(p.out) +
+                (((int64_t)seq * p.num_heads + head) * D + d0) * 2;
+    uint32_t w2[SL / 2];
 #pragma unroll
-    for (int ee = 0; ee < n_e; ++ee) {
-      const int d0 = (4 * r + e_lo + ee) * NDT;
-      uint32_t w[NDT / 2];
+    for (int k = 0; k < SL / 2; ++k) w2[k] = pack2<QT>(o[2 * k] * inv, o[2 * k + 1] * inv);
+    if constexpr (SL % 8 == 0) {
 #pragma unroll
-      for (int q2 = 0; q2 < NDT / 2; ++q2)
-        w[q2] = pack2<QT>(o[ee * NDT + 2 * q2] * inv, o[ee * NDT + 2 * q2 + 1] * inv);
-      if constexpr (NDT == 8) {
-        u32x4 v = {w[0], w[1], w[2], w[3]};
-        *reinterpret_cast<u32x4 *>(dst + d0 * 2) = v;
-      } else {
-        u32x2 v = {w[0], w[1]};
-        *reinterpret_cast<u32x2 *>(dst + d0 * 2) = v;
+      for (int k = 0; k < SL / 2; k += 4) {
+        u32x4 v = {w2[k], w2[k + 1], w2[k + 2], w2[k + 3]};
+        *reinterpret_cast<u32x4 *>(dst + k * 4) = v;
       }
+    } else if constexpr (SL % 4 == 0) {
+#pragma unroll
+      for (int k = 0; k < SL / 2; k += 2) {
+        u32x2 v = {w2[k], w2[k + 1]};
+        *reinterpret_cast<u32x2 *>(dst + k * 4) = v;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < SL / 2; ++k) *reinterpret_cast<uint32_t *>(dst + k * 4) = w2[k];
     }
   }
 }

@@ -21,9 +21,15 @@ constexpr int kMaxGroup = 16;
 //  * loop kernel: one work-group owns a whole (sequence, kv head); its wavefronts
 //    interleave 32-token chunks and merge once at the end through LDS.
 //  * split kernel: one work-group owns one partition of one (sequence, kv head).
+#ifndef FA_LOOP_WAVES
+#define FA_LOOP_WAVES 4
+#endif
+#ifndef FA_SPLIT_WAVES
+#define FA_SPLIT_WAVES 2
+#endif
 template <bool kPartitioned>
 struct WavesPerGroup {
-  static constexpr int value = kPartitioned ? 2 : 4;
+  static constexpr int value = kPartitioned ? FA_SPLIT_WAVES : FA_LOOP_WAVES;
 };
 
 // Reduce kernel: one wavefront per (sequence, head).
