@@ -7,6 +7,7 @@
 // here the same conditions become status codes because nothing may throw across a C ABI.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdint.h>
@@ -103,8 +104,8 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
     return fail(FA_ERR_BAD_SHAPE, "out, query, key_cache and value_cache must be 16-byte aligned");
   r->partition_size = s->partition_size > 0 ? s->partition_size : default_partition_size(s->head_size);
   if (split) {
-    if (r->partition_size % kChunkTokens)
-      return fail(FA_ERR_BAD_SHAPE, "partition_size %d must be a multiple of %d", r->partition_size, kChunkTokens);
+    if (r->partition_size % kMaxChunkTokens)
+      return fail(FA_ERR_BAD_SHAPE, "partition_size %d must be a multiple of %d", r->partition_size, kMaxChunkTokens);
     if (s->max_num_partitions <= 0 || s->max_num_partitions > 65535)
       return fail(FA_ERR_BAD_SHAPE, "max_num_partitions %d must be in [1, 65535]", s->max_num_partitions);
     if (max_context_len > 0 &&
@@ -155,22 +156,30 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   return p;
 }
 
-// Kernel-only time from a pair of events on the launch stream -- the counterpart of
-// upstream's get_exe_time (launch_kernels_loop.h:6-12), which reads SYCL event
-// profiling info.  Events are created once per thread and device and reused.
+// Kernel-only time -- the counterpart of upstream's get_exe_time
+// (launch_kernels_loop.h:6-12), which reads the start/end stamps of the kernel's own
+// SYCL event.  hipExtLaunchKernelGGL attaches a start and a stop event to the dispatch
+// itself, so the pair brackets the kernel and nothing else (events recorded with
+// separate hipEventRecord calls also count the gap between the record and the
+// dispatch).  Events are created once per thread and device and reused.
 class KernelTimer {
  public:
-  explicit KernelTimer(bool enabled, hipStream_t stream) : enabled_(enabled), stream_(stream) {}
-  hipError_t start(int slot) {
-    if (!enabled_) return hipSuccess;
-    hipError_t e = ensure();
-    if (e != hipSuccess) return e;
-    return hipEventRecord(events()[2 * slot], stream_);
+  KernelTimer(bool enabled, hipStream_t stream) : enabled_(enabled), stream_(stream) {}
+
+  // Launch `kernel` on the stream; with timing on, events 2*slot / 2*slot+1 bracket it.
+  template <typename Params>
+  hipError_t launch(void (*kernel)(Params), dim3 grid, dim3 block, int slot, const Params &prm) {
+    hipEvent_t start = nullptr, stop = nullptr;
+    if (enabled_) {
+      hipError_t e = ensure();
+      if (e != hipSuccess) return e;
+      start = events()[2 * slot];
+      stop = events()[2 * slot + 1];
+    }
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream_, start, stop, 0, prm);
+    return hipGetLastError();
   }
-  hipError_t stop(int slot) {
-    if (!enabled_) return hipSuccess;
-    return hipEventRecord(events()[2 * slot + 1], stream_);
-  }
+
   hipError_t read(int slot, float *us) {
     if (!enabled_) return hipSuccess;
     hipError_t e = hipEventSynchronize(events()[2 * slot + 1]);

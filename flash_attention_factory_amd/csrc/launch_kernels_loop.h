@@ -24,11 +24,9 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
                                         block_tables, context_lens, scale, shape, r);
   const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
-  FA_HIP_CHECK(timer.start(0));
-  hipLaunchKernelGGL((paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW>), grid, dim3(NW * 64), 0,
-                     r.stream, p);
-  FA_HIP_CHECK(hipGetLastError());
-  FA_HIP_CHECK(timer.stop(0));
+  FA_HIP_CHECK(timer.launch(
+      paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ, (FA_LPT != 0), Pipeline<KV8>::tiles_per_chunk>, grid,
+      dim3(NW * 64), 0, p));
   if (r.elapsed_us) FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
   return FA_OK;
 }

@@ -30,11 +30,9 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // sequence's length return at once and write nothing
   // (paged_attention_kernel_v2.hpp:577-579 does the same)
   const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
-  FA_HIP_CHECK(timer.start(0));
-  hipLaunchKernelGGL((paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW>), grid, dim3(NW * 64), 0,
-                     r.stream, p);
-  FA_HIP_CHECK(hipGetLastError());
-  FA_HIP_CHECK(timer.stop(0));
+  FA_HIP_CHECK(timer.launch(
+      paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ, false, Pipeline<KV8>::tiles_per_chunk>, grid,
+      dim3(NW * 64), 0, p));
 
   // kernel 2: one wavefront per (head, sequence)
   ReduceParams rp;
@@ -47,11 +45,8 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   rp.max_num_partitions = shape.max_num_partitions;
   rp.partition_size = r.partition_size;
   rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
-  FA_HIP_CHECK(timer.start(1));
-  hipLaunchKernelGGL((paged_attn_reduce_kernel<HEAD_SIZE, QT>), dim3(shape.num_heads, shape.num_seqs),
-                     dim3(kReduceThreads), 0, r.stream, rp);
-  FA_HIP_CHECK(hipGetLastError());
-  FA_HIP_CHECK(timer.stop(1));
+  FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT>,
+                            dim3(shape.num_heads, shape.num_seqs), dim3(kReduceThreads), 1, rp));
   if (r.elapsed_us) {
     FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
     FA_HIP_CHECK(timer.read(1, &r.elapsed_us[1]));

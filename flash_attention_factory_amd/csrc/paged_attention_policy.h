@@ -5,10 +5,11 @@
 
 namespace fa {
 
-// Tokens one wavefront consumes per software-pipeline step: two 16-token MFMA
-// tiles of scores feed one 32-deep P.V MFMA.
-constexpr int kChunkTokens = 32;
+// One MFMA score tile covers 16 tokens; a chunk -- the unit of the software pipeline of
+// one wavefront -- is 2 or 4 tiles (two tiles of scores feed one 32-deep P.V MFMA).
+// Partition boundaries must fall on chunk boundaries of the largest chunk.
 constexpr int kTileTokens = 16;
+constexpr int kMaxChunkTokens = 64;
 
 // Upstream partition sizes: 512 tokens for head size 128, 256 for head size 64
 // (paged_attention_policy_v2.hpp:28,50; the tests mirror it, test_paged.py:411-412).
@@ -22,17 +23,51 @@ constexpr int kMaxGroup = 16;
 //    interleave 32-token chunks and merge once at the end through LDS.
 //  * split kernel: one work-group owns one partition of one (sequence, kv head).
 #ifndef FA_LOOP_WAVES
-#define FA_LOOP_WAVES 4
+#define FA_LOOP_WAVES 8
 #endif
 #ifndef FA_SPLIT_WAVES
-#define FA_SPLIT_WAVES 2
+#define FA_SPLIT_WAVES 1
 #endif
 template <bool kPartitioned>
 struct WavesPerGroup {
   static constexpr int value = kPartitioned ? FA_SPLIT_WAVES : FA_LOOP_WAVES;
 };
 
-// Reduce kernel: one wavefront per (sequence, head).
-constexpr int kReduceThreads = 64;
+// Streaming pipeline of the attention kernel and the occupancy it is compiled for.
+//   PIPE 0: two register sets, the whole next chunk in flight under the current one.
+//   PIPE 1: one register set, K and V refilled separately right after their MFMAs.
+//   OCC   : wavefronts per SIMD the register allocator must fit (4 SIMDs per CU).
+#ifndef FA_PIPE
+#define FA_PIPE 1
+#endif
+#ifndef FA_OCC
+#define FA_OCC 3
+#endif
+#ifndef FA_PIPE_FP8
+#define FA_PIPE_FP8 FA_PIPE
+#endif
+#ifndef FA_OCC_FP8
+#define FA_OCC_FP8 FA_OCC
+#endif
+#ifndef FA_TPC
+#define FA_TPC 2
+#endif
+#ifndef FA_TPC_FP8
+#define FA_TPC_FP8 2
+#endif
+template <bool kKV8>
+struct Pipeline {
+  static constexpr int pipe = kKV8 ? FA_PIPE_FP8 : FA_PIPE;
+  static constexpr int occ = kKV8 ? FA_OCC_FP8 : FA_OCC;
+  static constexpr int tiles_per_chunk = kKV8 ? FA_TPC_FP8 : FA_TPC;
+};
+
+// Longest-sequence-first assignment of sequences to work-groups (loop kernel).
+#ifndef FA_LPT
+#define FA_LPT 0
+#endif
+
+// Reduce kernel: four wavefronts per (sequence, head).
+constexpr int kReduceThreads = 256;
 
 }  // namespace fa

@@ -6,9 +6,12 @@
 //   out = sum_p (w_p / sum_q w_q) * tmp_out[p, :]      (compute_out :771-864, collect_out :868-934)
 // Only the ceil(context_len / partition_size) live partitions are read (:679,716).
 //
-// One wavefront per (sequence, head): lane j owns D/64 consecutive output elements, so
-// every tmp_out row is read with one fully coalesced wave load; partition weights are
-// computed 64 at a time, one per lane, and broadcast with lane shuffles.
+// One work-group of four wavefronts per (sequence, head).  The kernel is a chain of
+// dependent memory round trips, so it is built to have as few of them as possible:
+// wavefront w owns partitions w, w+4, w+8, ... and requests up to 16 of their tmp_out
+// rows (one coalesced 512-byte row per load) together with the partition scalars, before
+// anything is waited for; the weights are applied when both have arrived; the four
+// partial sums meet in LDS.  Lane j owns D/64 consecutive output elements.
 #pragma once
 
 #include "paged_attention_utils.h"
@@ -27,10 +30,15 @@ struct ReduceParams {
   int32_t max_context;  // max_blocks_per_seq * block_size: lengths are cut to it
 };
 
+constexpr int kReduceWaves = 4;
+constexpr int kReduceRowsInFlight = 16;  // per wavefront; 4 x 16 = 64 partitions per batch
+
 template <int D, typename QT>
-__global__ void __launch_bounds__(64) paged_attn_reduce_kernel(const ReduceParams p) {
+__global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
   constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
-  const int lane = threadIdx.x;
+  constexpr int R = kReduceRowsInFlight;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
   const int ctx = min(p.context_lens[seq], p.max_context);
@@ -42,46 +50,73 @@ __global__ void __launch_bounds__(64) paged_attn_reduce_kernel(const ReduceParam
   const float *es = p.exp_sums + base;
   const float *tmp = p.tmp_out + base * D + lane * EPL;
 
-  float M = -INFINITY;
-  for (int q = lane; q < np; q += 64) M = fmaxf(M, ml[q]);
+  // first batch of rows and the scalars go out together
+  float v[R][EPL];
+#pragma unroll
+  for (int u = 0; u < R; ++u) {
+    const int q = wave + kReduceWaves * u;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * D + e] : 0.f;
+  }
+  // lane q keeps the scalars of partition q (first 64 partitions) in registers
+  const float ml0 = (lane < np) ? ml[lane] : -INFINITY;
+  const float es0 = (lane < np) ? es[lane] : 0.f;
+  float M = ml0;
+  for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q]);
   M = wave_max(M);
+  float w_lane = es0 * __expf(ml0 - M);  // weight of partition `lane`
+  float W = w_lane;
 
   float acc[EPL];
 #pragma unroll
   for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
-  float W = 0.f;
-  for (int q0 = 0; q0 < np; q0 += 64) {
-    const int q = q0 + lane;
-    const float w_lane = (q < np) ? es[q] * __expf(ml[q] - M) : 0.f;
-    W += w_lane;
-    const int cnt = min(64, np - q0);
-    int j = 0;
-    for (; j + 4 <= cnt; j += 4) {  // four rows in flight
-      float v[4][EPL];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+  for (int u = 0; u < R; ++u) {
+    const int q = wave + kReduceWaves * u;  // wave-uniform, < 64
+    const float w = __shfl(w_lane, q);      // 0 for q >= np
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) v[u][e] = tmp[(int64_t)(q0 + j + u) * D + e];
+    for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
+  }
+  // contexts beyond 64 partitions: further batches of 64 partitions
+  for (int q0 = kReduceWaves * R; q0 < np; q0 += kReduceWaves * R) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float w = __shfl(w_lane, j + u);
+    for (int u = 0; u < R; ++u) {
+      const int q = q0 + wave + kReduceWaves * u;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
-      }
+      for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * D + e] : 0.f;
     }
-    for (; j < cnt; ++j) {
-      const float w = __shfl(w_lane, j);
+    const int ql = q0 + lane;
+    w_lane = (ql < np) ? es[ql] * __expf(ml[ql] - M) : 0.f;
+    W += w_lane;
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) acc[e] += w * tmp[(int64_t)(q0 + j) * D + e];
+    for (int u = 0; u < R; ++u) {
+      const float w = __shfl(w_lane, wave + kReduceWaves * u);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
     }
   }
   W = wave_sum(W);
+
+  __shared__ float part[kReduceWaves][D];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) part[wave][lane * EPL + e] = acc[e];
+  __syncthreads();
+  if (wave != 0) return;
   const float inv = 1.0f / W;
-  char *dst = reinterpret_cast<char *>(p.out) + (((int64_t)seq * p.num_heads + head) * D + lane * EPL) * 2;
+  float o[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    float a = 0.f;
+#pragma unroll
+    for (int w = 0; w < kReduceWaves; ++w) a += part[w][lane * EPL + e];
+    o[e] = a * inv;
+  }
+  char *dst = reinterpret_cast<char *>(p.out) +
+              (((int64_t)seq * p.num_heads + head) * D + lane * EPL) * 2;
   if constexpr (EPL == 2) {
-    *reinterpret_cast<uint32_t *>(dst) = pack2<QT>(acc[0] * inv, acc[1] * inv);
+    *reinterpret_cast<uint32_t *>(dst) = pack2<QT>(o[0], o[1]);
   } else {
-    const uint32_t w = pack2<QT>(acc[0] * inv, 0.f);
+    const uint32_t w = pack2<QT>(o[0], 0.f);
     *reinterpret_cast<uint16_t *>(dst) = (uint16_t)(w & 0xffffu);
   }
 }

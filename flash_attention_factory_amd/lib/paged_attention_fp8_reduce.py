@@ -3,15 +3,17 @@
 Drop-in for the upstream extension module of the same name
 (paged_attention_fp8_reduce/paged_attention_fp8_reduce.cpp:21-39,84-86): same positional arguments, same return value
 (a list of kernel times in microseconds).  ``timed=False`` (keyword only, not in
-upstream) launches asynchronously on the current stream and returns ``[]``.
+upstream) launches asynchronously on the current stream and returns ``[]``;
+``partition_size`` (keyword only) overrides the upstream policy value (512 tokens for
+head size 128, 256 for head size 64).
 """
 from ._run import run_impl
 
 
 def run(max_logits, exp_sums, tem_output, output, debug_output, query, key_cache, value_cache,
         block_tables, context_lens, num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
-        alibi_slopes, sinks, softcap, *, timed=True):
+        alibi_slopes, sinks, softcap, *, timed=True, partition_size=0):
     return run_impl("fa_paged_attention_fp8_reduce", True, True, max_logits, exp_sums, tem_output, output,
                     debug_output, query, key_cache, value_cache, block_tables, context_lens,
                     num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
-                    alibi_slopes, sinks, softcap, timed=timed)
+                    alibi_slopes, sinks, softcap, timed=timed, partition_size=partition_size)

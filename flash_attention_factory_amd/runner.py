@@ -64,6 +64,9 @@ def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
     head = (bufs.max_logits, bufs.exp_sums, bufs.tmp_out, bufs.out, bufs.debug, w.query, kc, vc,
             w.block_tables, w.context_lens, G, w.scale)
     tail = (w.block_size, max_ctx, bufs.alibi, w.sinks, -1.0)
+    kw = dict(timed=timed)
+    if "reduce" in kernel:
+        kw["partition_size"] = w.partition_size
     if w.is_fp8:
-        return mod.run(*head, w.fp8_scale, *tail, timed=timed)
-    return mod.run(*head, *tail, timed=timed)
+        return mod.run(*head, w.fp8_scale, *tail, **kw)
+    return mod.run(*head, *tail, **kw)
