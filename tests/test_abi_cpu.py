@@ -1,0 +1,122 @@
+"""CPU-only checks of the C ABI: the library loads, exports every function the header
+declares, and rejects bad arguments with the documented status codes (validate_only
+launches nothing, so no GPU is needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from flash_attention_factory_amd import _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    if not os.path.exists(_cabi.LIBRARY):
+        from flash_attention_factory_amd import _build
+        _build.build()
+    return _cabi.load()
+
+
+def test_header_symbols_are_exported(L):
+    header = open(os.path.join(ROOT, "include", "fa_paged_attention.h")).read()
+    body = header[header.index('extern "C"'):]
+    declared = set(re.findall(r"\b(fa_[a-z0-9_]+)\s*\(", body))
+    assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.fa_paged_attention_abi_version() == 1
+
+
+def test_struct_layouts_match_header():
+    # field order and sizes of the two structs as the header lays them out
+    assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
+    assert _cabi.Shape.kv_block_stride.offset == 32
+    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4
+    assert _cabi.Options.elapsed_us.offset == 32
+
+
+def _shape(**kw):
+    s = _cabi.Shape()
+    base = dict(num_seqs=2, num_heads=8, num_kv_heads=2, head_size=128, block_size=16,
+                max_blocks_per_seq=4, max_num_partitions=1, partition_size=0,
+                kv_block_stride=2 * 16 * 128, kv_token_stride=128, kv_head_stride=16 * 128,
+                q_dtype=_cabi.FA_DTYPE_F16, num_pool_blocks=8)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(s, k, v)
+    return s
+
+
+def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0):
+    op = _cabi.Options()
+    op.validate_only = 1
+    name = "fa_paged_attention_" + ("fp8_" if fp8 else "") + ("reduce" if split else "loop")
+    args = [ptr, ptr, ptr, ptr, ptr, ptr, 0.1, max_ctx]
+    if split:
+        args += [scratch, scratch, scratch]
+    sh = shape or _shape()
+    return getattr(L, name)(*args, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_valid_arguments_pass(L, split, fp8):
+    rc, msg = _call(L, split, fp8)
+    assert rc == _cabi.FA_OK and msg == ""
+
+
+def test_error_codes(L):
+    assert _call(L, ptr=0)[0] == _cabi.FA_ERR_NULL_POINTER
+    assert _call(L, split=True, scratch=0)[0] == _cabi.FA_ERR_NULL_POINTER
+    rc, msg = _call(L, shape=_shape(head_size=96))
+    assert rc == _cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE and "Unsupported head size or block size" in msg
+    assert _call(L, shape=_shape(block_size=24))[0] == _cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE
+    assert _call(L, shape=_shape(block_size=8))[0] == _cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE
+    rc, msg = _call(L, shape=_shape(num_heads=7))
+    assert rc == _cabi.FA_ERR_UNSUPPORTED_GROUP and "Unsupported number of queries per token" in msg
+    assert _call(L, shape=_shape(num_heads=34, num_kv_heads=2))[0] == _cabi.FA_ERR_UNSUPPORTED_GROUP
+    assert _call(L, shape=_shape(q_dtype=5))[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
+    assert _call(L, shape=_shape(num_seqs=0))[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _call(L, shape=_shape(kv_token_stride=100))[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _call(L, ptr=0x1008)[0] == _cabi.FA_ERR_BAD_SHAPE
+    # 4 blocks of 16 tokens cannot hold 100 tokens
+    assert _call(L, max_ctx=100)[0] == _cabi.FA_ERR_BAD_SHAPE
+    # split path: one partition of 512 tokens cannot hold 600
+    rc, msg = _call(L, split=True, shape=_shape(max_blocks_per_seq=64), max_ctx=600)
+    assert rc == _cabi.FA_ERR_PARTITION_OVERFLOW and "partitions" in msg
+    assert _call(L, split=True, shape=_shape(partition_size=48))[0] == _cabi.FA_ERR_BAD_SHAPE
+    # the same shape is fine for the loop entry, which has no partitions
+    assert _call(L, shape=_shape(partition_size=48))[0] == _cabi.FA_OK
+    # NULL shape / NULL options
+    op = _cabi.Options(); op.validate_only = 1
+    assert L.fa_paged_attention_loop(1, 1, 1, 1, 1, 1, 0.1, 0, None, ctypes.byref(op)) == _cabi.FA_ERR_NULL_POINTER
+
+
+def test_run_shim_rejects_cpu_tensors():
+    import torch
+    from flash_attention_factory_amd import runner, workloads as W
+    w = W.make_config(0)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        runner.run_workload(w, "loop")
+
+
+def test_workload_generators_are_deterministic():
+    import torch
+    from flash_attention_factory_amd import workloads as W
+    a, b = W.make_config(0), W.make_config(0)
+    assert torch.equal(a.query, b.query) and torch.equal(a.key_cache, b.key_cache)
+    assert torch.equal(a.block_tables, b.block_tables) and torch.equal(a.context_lens, b.context_lens)
+    # every sequence's blocks are distinct pool blocks, no block shared between sequences
+    used = []
+    for s in range(a.num_seqs):
+        nb = (int(a.context_lens[s]) + a.block_size - 1) // a.block_size
+        used += a.block_tables[s, :nb].tolist()
+    assert len(used) == len(set(used)) and max(used) < a.key_cache.shape[0]
+    assert a.algorithmic_bytes() == int(a.context_lens.sum()) * 8 * 64 * 2 * 2 + 2 * 4 * 8 * 64 * 2 + \
+        sum((int(n) + 15) // 16 for n in a.context_lens) * 4 + 4 * 4
+    g = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=64, seqlen_k=339, varlen=True, has_sinks=True)
+    assert g.partition_size == 256 and g.key_cache.shape == (12, 64, 2, 64)
+    assert int(g.context_lens.min()) >= 319 and int(g.context_lens.max()) <= 339
