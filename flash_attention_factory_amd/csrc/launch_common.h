@@ -15,6 +15,7 @@
 
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
+#include "paged_attention_persistent_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
 
@@ -143,7 +144,9 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.sinks = r.sinks;
   p.score_scale_log2 = scale * r.fp8_scale * kLog2e;
   p.out_scale = r.fp8_scale;
+  p.num_seqs = s.num_seqs;
   p.num_heads = s.num_heads;
+  p.num_kv_heads = s.num_kv_heads;
   p.group = r.group;
   p.max_blocks_per_seq = s.max_blocks_per_seq;
   p.max_num_partitions = s.max_num_partitions;
@@ -154,6 +157,27 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;
   return p;
+}
+
+// How many work-groups of a single-wavefront kernel the current device keeps resident
+// (compute units x work-groups per compute unit).  Asked once per kernel and device.
+template <typename K>
+inline hipError_t resident_wavefronts(K kernel, int *out) {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev != cached_dev) {
+    int cus = 0, per_cu = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64, 0);
+    if (e != hipSuccess) return e;
+    cached = cus * (per_cu > 0 ? per_cu : 1);
+    cached_dev = dev;
+  }
+  *out = cached;
+  return hipSuccess;
 }
 
 // Kernel-only time -- the counterpart of upstream's get_exe_time

@@ -26,13 +26,26 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   const PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache,
                                         value_cache, block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
-  // kernel 1: one work-group per (kv head, partition, sequence); partitions past a
-  // sequence's length return at once and write nothing
-  // (paged_attention_kernel_v2.hpp:577-579 does the same)
-  const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
-  FA_HIP_CHECK(timer.launch(
-      paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ, false, Pipeline<KV8>::tiles_per_chunk>, grid,
-      dim3(NW * 64), 0, p));
+  // kernel 1.  Persistent form when the batch fits it: as many single-wavefront
+  // work-groups as the GPU keeps resident walk the list of live partitions.  Otherwise
+  // one work-group per (kv head, partition slot, sequence); slots past a sequence's
+  // length return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
+  if (kUsePersistentSplit && shape.num_seqs <= kPersistentMaxSeqs && shape.num_pool_blocks > 0) {
+    auto kernel = paged_attn_split_persistent_kernel<HEAD_SIZE, QT, KV8, Pipeline<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk>;
+    int resident = 0;
+    FA_HIP_CHECK(resident_wavefronts(kernel, &resident));
+    const int64_t max_items =
+        (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
+    const dim3 grid((unsigned)std::min<int64_t>(resident, max_items));
+    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(64), 0, p));
+  } else {
+    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+    FA_HIP_CHECK(timer.launch(
+        paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ,
+                          false, Pipeline<KV8>::tiles_per_chunk>,
+        grid, dim3(NW * 64), 0, p));
+  }
 
   // kernel 2: one wavefront per (head, sequence)
   ReduceParams rp;

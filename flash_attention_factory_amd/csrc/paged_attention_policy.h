@@ -62,6 +62,12 @@ struct Pipeline {
   static constexpr int tiles_per_chunk = kKV8 ? FA_TPC_FP8 : FA_TPC;
 };
 
+// Split path: use the persistent attention kernel when the batch allows it.
+#ifndef FA_PERSISTENT_SPLIT
+#define FA_PERSISTENT_SPLIT 1
+#endif
+constexpr bool kUsePersistentSplit = FA_PERSISTENT_SPLIT != 0;
+
 // Longest-sequence-first assignment of sequences to work-groups (loop kernel).
 #ifndef FA_LPT
 #define FA_LPT 0

@@ -127,7 +127,31 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Load one int32 of read-only input through the scalar unit.  `p` must be wave-uniform and
+// must point at memory the kernel never writes (block tables, context lengths): the
+// constant address space tells the compiler exactly that, so the load stays a scalar load
+// even when the kernel has stored to other buffers before it.
+__device__ __forceinline__ int32_t load_uniform_i32(const int32_t *p) {
+  typedef const int32_t __attribute__((address_space(4))) *const_ptr;
+  return *(const_ptr)(uintptr_t)p;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// K/V bytes are read exactly once per launch: FA_STREAM_LOADS marks those loads
+// non-temporal so they do not displace the few lines that are re-used (queries, block
+// tables, the split path's scratch).
+#ifndef FA_STREAM_LOADS
+#define FA_STREAM_LOADS 0
+#endif
+template <typename T>
+__device__ __forceinline__ T stream_load(const T *p) {
+#if FA_STREAM_LOADS
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
 
 // Global loads of 4, 8 or 16 bytes per lane.
 template <int DWORDS>
@@ -135,21 +159,21 @@ struct VLoad;
 template <>
 struct VLoad<4> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[4], const char *p) {
-    u32x4 t = *reinterpret_cast<const u32x4 *>(p);
+    u32x4 t = stream_load(reinterpret_cast<const u32x4 *>(p));
     dst[0] = t[0]; dst[1] = t[1]; dst[2] = t[2]; dst[3] = t[3];
   }
 };
 template <>
 struct VLoad<2> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[2], const char *p) {
-    u32x2 t = *reinterpret_cast<const u32x2 *>(p);
+    u32x2 t = stream_load(reinterpret_cast<const u32x2 *>(p));
     dst[0] = t[0]; dst[1] = t[1];
   }
 };
 template <>
 struct VLoad<1> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[1], const char *p) {
-    dst[0] = *reinterpret_cast<const uint32_t *>(p);
+    dst[0] = stream_load(reinterpret_cast<const uint32_t *>(p));
   }
 };
 

@@ -1,0 +1,330 @@
+// One wavefront's share of paged-attention decode on gfx950: operand loads, the two
+// MFMA products and the online softmax between them.  The grid kernel and the
+// persistent kernel are both built from this.
+//
+// Per chunk of TPC 16-token tiles (the query group's G <= 16 heads are the 16 MFMA columns):
+//   S^T[token, head] = K[token, :] . Q^T[:, head]      per tile: D/32 MFMA 16x16x32
+//   online softmax over tokens, fp32, base 2            VALU + two cross-row shuffles
+//   O^T[d, head]    += V^T[d, token] . P^T[token, head] per 32 tokens: D/16 MFMA 16x16x32
+// K rows enter the MFMA "A" operand exactly as they lie in HBM (lane 16r+i loads 16 B
+// of token i); V rows are loaded row-wise (16 lanes cover one token row) and
+// transposed inside each lane with byte permutes, so neither needs LDS.  The scores
+// come out of the first MFMA in the register layout the second MFMA wants for P^T.
+//
+// Arithmetic follows the upstream kernels (scores paged_attention_kernel_loop.hpp:227-348,
+// softmax :353-444, P.V :455-546; FP8 paged_attention_kernel_fp8_loop.hpp:328-333,540-545):
+// fp32 scores scaled after the dot, tail tokens masked to -inf, probabilities rounded to
+// the query dtype before P.V, fp8_scale folded into the score scale and the final scale.
+#pragma once
+
+#include <type_traits>
+
+#include "paged_attention_policy.h"
+#include "paged_attention_utils.h"
+
+#ifndef FA_STREAM_STORES
+#define FA_STREAM_STORES 0
+#endif
+
+namespace fa {
+
+struct PagedAttnParams {
+  void *out;              // loop: [S,H,D] q dtype.  split: tmp_out [S,H,NP,D] fp32
+  float *exp_sums;        // split only: [S,H,NP]
+  float *max_logits;      // split only: [S,H,NP]
+  const void *query;      // [S,H,D]
+  const char *key_cache;
+  const char *value_cache;
+  const int32_t *block_tables;  // [S,MB]
+  const int32_t *context_lens;  // [S]
+  const void *sinks;            // [H] q dtype or nullptr
+  float score_scale_log2;       // sm_scale * fp8_scale * log2(e)
+  float out_scale;              // fp8_scale (1 for 16-bit caches)
+  int32_t num_seqs;
+  int32_t num_heads;
+  int32_t num_kv_heads;
+  int32_t group;                // query heads per kv head
+  int32_t max_blocks_per_seq;
+  int32_t max_num_partitions;
+  int32_t partition_size;       // tokens; multiple of 64
+  int32_t block_shift;          // log2(block_size)
+  int32_t max_block_id;         // block ids are clamped into [0, max_block_id]
+  int64_t kv_block_bytes;       // strides in BYTES
+  int64_t kv_token_bytes;
+  int64_t kv_head_bytes;
+};
+
+// TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
+// pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
+template <int D, typename QT, bool KV8, int TPC>
+struct WaveAttn {
+  static_assert(TPC == 2 || TPC == 4, "a chunk is one or two 32-token P.V steps");
+  static constexpr int ROWB = D * (KV8 ? 1 : 2);  // bytes per token row
+  static constexpr int KL = ROWB / 64;            // 16-byte K loads per lane and tile
+  static constexpr int KSTEPS = D / 32;           // MFMA k-steps across the head dimension
+  static constexpr int NDT = D / 16;  // output d-tiles; lane row i of tile dt is d = i*NDT + dt
+  static constexpr int VW = ROWB / 64;            // dwords of V per lane and token
+  static constexpr int VB = VW * 4;               // bytes of V per lane and token
+  static constexpr int CT = TPC * kTileTokens;    // tokens per chunk
+  static constexpr int NP2 = TPC / 2;             // 32-token P.V steps per chunk
+  static constexpr int NR = NDT * 4;              // accumulator values per lane
+
+  // Register image of one chunk of K and V.
+  struct Chunk {
+    u32x4 k[TPC][KL];
+    uint32_t v[4 * TPC][VW];
+  };
+  struct Ids { int v[TPC]; };      // physical block id of every tile of a chunk
+  struct Scores { f32x4 v[TPC]; };
+  struct Probs { u32x4 v[NP2]; };
+
+  const PagedAttnParams &p;
+  const int r;  // 16-lane row of the wavefront
+  const int i;  // position in the row: token (K), head (Q, P, O) or d-row (V)
+  const int blk_mask;
+
+  // Q^T as the MFMA "B" operand, one dword quad per k-step.  k-slot (r, e) of step c
+  // stands for head-dim element qd(c, r) + e; K uses the same map.
+  u32x4 qB[KSTEPS];
+  // Online softmax state.  m: running max (base-2 units) of head i, identical in the four
+  // rows r.  l: this lane's share of the running sum (its own tokens).
+  // acc[dt][e]: O^T[d = (4r+e)*NDT + dt][head i], un-normalised.
+  float m, l;
+  f32x4 acc[NDT];
+
+  __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
+      : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {}
+
+  __device__ __forceinline__ void load_q(int seq, int kvh) {
+    const int head = kvh * p.group + i;
+    const char *qrow = reinterpret_cast<const char *>(p.query) +
+                       ((int64_t)seq * p.num_heads + head) * (D * 2);
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c) {
+      const int d0 = KV8 ? ((c >> 1) * 4 + r) * 16 + (c & 1) * 8 : (c * 4 + r) * 8;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qB[c] = (i < p.group) ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
+    }
+  }
+
+  // The sink is one more logit with a zero value row; it belongs to the wavefront that
+  // owns the start of the context (paged_attention_kernel_loop.hpp:387-391,
+  // paged_attention_kernel_v2.hpp:373-376).  load_sink only requests the 16-bit value
+  // (kNoSink if there is none for this lane); reset() decodes it, so that nothing has to
+  // wait for the load where it is issued.
+  static constexpr uint32_t kNoSink = 0xffffffffu;
+  __device__ __forceinline__ uint32_t load_sink(int kvh, bool with_sink) const {
+    uint32_t raw = kNoSink;
+    if (with_sink && p.sinks != nullptr && i < p.group)
+      raw = *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(p.sinks) +
+                                                (kvh * p.group + i) * 2);
+    return raw;
+  }
+
+  // Fresh softmax state, optionally seeded with a sink logit (weight 1, value row 0).
+  __device__ __forceinline__ void reset(uint32_t sink_raw) {
+    m = -INFINITY;
+    l = 0.f;
+    if (sink_raw != kNoSink) {
+      const uint16_t h = (uint16_t)sink_raw;
+      m = load_scalar16<QT>(&h) * kLog2e;
+      l = (r == 0) ? 1.f : 0.f;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Physical block id of every 16-token tile of chunk ci of a sequence's table row.
+  // Columns are clamped to `col_max` and ids into the pool, so a tile wholly past the
+  // context re-reads memory that exists; it is masked later.
+  __device__ __forceinline__ Ids fetch_ids(const int32_t *table, int ci, int col_max) const {
+    Ids ids;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) {
+      const int col = min((ci * CT + t * kTileTokens) >> p.block_shift, col_max);
+      ids.v[t] = min((uint32_t)load_uniform_i32(table + col), (uint32_t)p.max_block_id);
+    }
+    return ids;
+  }
+
+  __device__ __forceinline__ int64_t tile_offset(int kvh, int ci, int t, const Ids &ids) const {
+    return (int64_t)ids.v[t] * p.kv_block_bytes + (int64_t)kvh * p.kv_head_bytes +
+           (int64_t)((ci * CT + t * kTileTokens) & blk_mask) * p.kv_token_bytes;
+  }
+
+  // K and V of a chunk go out separately so that either half of the register set can be
+  // refilled as soon as it has been consumed.
+  __device__ __forceinline__ void issue_k(Chunk &R, int kvh, int ci, const Ids &ids) const {
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) {
+      const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
+#pragma unroll
+      for (int c = 0; c < KL; ++c) R.k[t][c] = stream_load(reinterpret_cast<const u32x4 *>(kp + c * 64));
+    }
+  }
+  __device__ __forceinline__ void issue_v(Chunk &R, int kvh, int ci, const Ids &ids) const {
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) {
+      const char *vp = p.value_cache + tile_offset(kvh, ci, t, ids) +
+                       (int64_t)(4 * r) * p.kv_token_bytes + i * VB;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) VLoad<VW>::ld(R.v[t * 4 + e], vp + e * p.kv_token_bytes);
+    }
+  }
+
+  // K "A" operand of k-step c for one tile: row i = token, 8 head-dim elements.
+  __device__ __forceinline__ u32x4 k_operand(const Chunk &R, int tile, int c) const {
+    if constexpr (!KV8) {
+      return R.k[tile][c];
+    } else {
+      const u32x4 src = R.k[tile][c >> 1];
+      const int h = c & 1;
+      u32x4 o;
+      o[0] = e5m2_adjacent_pair<QT>(src[2 * h], 0);
+      o[1] = e5m2_adjacent_pair<QT>(src[2 * h], 1);
+      o[2] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 0);
+      o[3] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 1);
+      return o;
+    }
+  }
+
+  // V^T "A" operand of d-tile dt for the 32-token step `pr` of the chunk: row i = d-row,
+  // k-slots = this lane row's 8 tokens of the step.  In-lane transpose: R.v[e] holds
+  // token e's NDT consecutive head-dim elements.
+  __device__ __forceinline__ u32x4 v_operand(const Chunk &R, int pr, int dt) const {
+    u32x4 o;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int e0 = pr * 8 + 2 * c;
+      if constexpr (!KV8) {
+        const uint32_t y = R.v[e0][dt >> 1], x = R.v[e0 + 1][dt >> 1];
+        o[c] = (dt & 1) ? ((y >> 16) | (x & 0xffff0000u)) : ((y & 0xffffu) | (x << 16));
+      } else {
+        const uint32_t y = (R.v[e0][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
+        const uint32_t x = (R.v[e0 + 1][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
+        o[c] = e5m2_pair<QT>(y, x);
+      }
+    }
+    return o;
+  }
+
+  // scores: S^T tile rows are tokens 4r+e of the tile, column i is the head
+  __device__ __forceinline__ Scores qk(const Chunk &R) const {
+    Scores s;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) s.v[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c)
+#pragma unroll
+      for (int t = 0; t < TPC; ++t) s.v[t] = mfma_16x16x32<QT>(k_operand(R, t, c), qB[c], s.v[t]);
+    return s;
+  }
+
+  // Online softmax step over the chunk's tokens; returns the P^T "B" operands.
+  // check_tail: whether this chunk can reach past tok_end (a compile-time false drops
+  // the masking code from the steady-state loop).
+  template <bool CHECK_TAIL>
+  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end) {
+    constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
+    float t[NT];
+#pragma unroll
+    for (int e = 0; e < NT; ++e) t[e] = s.v[e >> 2][e & 3] * p.score_scale_log2;
+    if constexpr (CHECK_TAIL) {
+      const int t0 = ci * CT;
+      if (t0 + CT > tok_end) {  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < NT; ++e) {
+          const int tok = t0 + (e >> 2) * kTileTokens + 4 * r + (e & 3);
+          if (tok >= tok_end) {
+            t[e] = -INFINITY;  // select, never multiply: the pool may hold NaN there
+#pragma unroll
+            for (int w = 0; w < VW; ++w) R.v[e][w] = 0u;
+          }
+        }
+      }
+    }
+    float mx = t[0];
+#pragma unroll
+    for (int e = 1; e < NT; ++e) mx = fmaxf(mx, t[e]);
+    mx = rows_max(mx);
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2(m - m_new);  // exp2(-inf) = 0 on the first chunk
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < NT; ++e) {
+      t[e] = fast_exp2(t[e] - m_new);
+      ps += t[e];
+    }
+    l = l * alpha + ps;
+    m = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+    }
+    // k-slots (r, e) of step pr = this lane's eight tokens of the step, rounded to the q
+    // dtype (paged_attention_kernel_loop.hpp:404-407)
+    Probs pb;
+#pragma unroll
+    for (int pr = 0; pr < NP2; ++pr)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) pb.v[pr][c] = pack2<QT>(t[pr * 8 + 2 * c], t[pr * 8 + 2 * c + 1]);
+    return pb;
+  }
+
+  __device__ __forceinline__ void pv(const Chunk &R, const Probs &pb) {
+#pragma unroll
+    for (int pr = 0; pr < NP2; ++pr)
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        acc[dt] = mfma_16x16x32<QT>(v_operand(R, pr, dt), pb.v[pr], acc[dt]);
+  }
+
+  // A lane's NR accumulator values are NR consecutive head-dim elements of head i:
+  // d = 4r*NDT + idx with idx = e*NDT + dt.
+  __device__ __forceinline__ float acc_at(int idx) const { return acc[idx % NDT][idx / NDT]; }
+
+  // Store `n` normalised fp32 values starting at head-dim element d0 of one tmp_out row.
+  template <int N>
+  static __device__ __forceinline__ void store_f32(float *dst, const float (&o)[N], float inv) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        f32x4 v = {o[k] * inv, o[k + 1] * inv, o[k + 2] * inv, o[k + 3] * inv};
+#if FA_STREAM_STORES
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst + k));
+#else
+        *reinterpret_cast<f32x4 *>(dst + k) = v;
+#endif
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; ++k) dst[k] = o[k] * inv;
+    }
+  }
+
+  // Store `n` normalised values rounded to the q dtype.
+  template <int N>
+  static __device__ __forceinline__ void store_q(char *dst, const float (&o)[N], float inv) {
+    uint32_t w2[N / 2];
+#pragma unroll
+    for (int k = 0; k < N / 2; ++k) w2[k] = pack2<QT>(o[2 * k] * inv, o[2 * k + 1] * inv);
+    if constexpr (N % 8 == 0) {
+#pragma unroll
+      for (int k = 0; k < N / 2; k += 4) {
+        u32x4 v = {w2[k], w2[k + 1], w2[k + 2], w2[k + 3]};
+        *reinterpret_cast<u32x4 *>(dst + k * 4) = v;
+      }
+    } else if constexpr (N % 4 == 0) {
+#pragma unroll
+      for (int k = 0; k < N / 2; k += 2) {
+        u32x2 v = {w2[k], w2[k + 1]};
+        *reinterpret_cast<u32x2 *>(dst + k * 4) = v;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < N / 2; ++k) *reinterpret_cast<uint32_t *>(dst + k * 4) = w2[k];
+    }
+  }
+};
+
+}  // namespace fa

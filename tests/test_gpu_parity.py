@@ -147,6 +147,35 @@ def test_edge_cases(oracle):
     torch.testing.assert_close(out[[1, 3]].float(), ref[[1, 3]].float(), atol=ATOL, rtol=RTOL)
 
 
+def test_large_batch_uses_grid_form_of_split_kernel(oracle):
+    """More than 256 sequences: the split path falls back from the persistent kernel to
+    one work-group per (kv head, partition slot, sequence)."""
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.randint(1, 700, (300,), generator=gen).tolist()
+    w = W.make_config(0, num_seqs=300, pool_blocks=300 * 44, lens=lens)
+    w.partition_size = 256
+    for kernel in ("reduce", "loop"):
+        bufs, _ = _run(w, kernel)
+        _check(bufs.out, w, oracle, f"300 sequences/{kernel}")
+
+
+def test_persistent_split_many_items_per_wavefront(oracle):
+    """Enough live partitions that every resident wavefront walks several items, with
+    sinks, ragged lengths and empty sequences in between."""
+    gen = torch.Generator().manual_seed(9)
+    lens = torch.randint(1, 3000, (200,), generator=gen)
+    lens[::7] = 0
+    w = W.make_config(0, num_seqs=200, pool_blocks=200 * 188, lens=lens.tolist())
+    w.partition_size = 256
+    w.sinks = torch.linspace(-2, 2, w.num_heads).to(w.query.dtype)
+    bufs, _ = _run(w, "reduce")
+    out = bufs.out.cpu()
+    assert (out[lens == 0] == 0).all()
+    ref = call_oracle(oracle.attention_ref, w)
+    live = lens > 0
+    torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
+
+
 def test_bf16_and_fp8_scale(oracle):
     # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
     w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,
