@@ -15,6 +15,7 @@
 
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
+#include "paged_attention_loop_persistent_kernel.h"
 #include "paged_attention_persistent_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
@@ -159,10 +160,10 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   return p;
 }
 
-// How many work-groups of a single-wavefront kernel the current device keeps resident
+// How many work-groups of `threads` threads of a kernel the current device keeps resident
 // (compute units x work-groups per compute unit).  Asked once per kernel and device.
 template <typename K>
-inline hipError_t resident_wavefronts(K kernel, int *out) {
+inline hipError_t resident_groups(K kernel, int threads, int *out) {
   static thread_local int cached_dev = -1, cached = 0;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -171,7 +172,7 @@ inline hipError_t resident_wavefronts(K kernel, int *out) {
     int cus = 0, per_cu = 0;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64, 0);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
     if (e != hipSuccess) return e;
     cached = cus * (per_cu > 0 ? per_cu : 1);
     cached_dev = dev;

@@ -7,6 +7,8 @@
 // 16-way switch of upstream collapses to head size x dtype.
 #pragma once
 
+#include <algorithm>
+
 #include "launch_common.h"
 
 namespace fa {
@@ -22,11 +24,25 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   constexpr int NW = WavesPerGroup<false>::value;
   const PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
                                         block_tables, context_lens, scale, shape, r);
-  const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
-  FA_HIP_CHECK(timer.launch(
-      paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ, (FA_LPT != 0), Pipeline<KV8>::tiles_per_chunk>, grid,
-      dim3(NW * 64), 0, p));
+  const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
+  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0) {
+    // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
+    // sequences first, with the next item's first loads issued before each merge.
+    constexpr int PW = PersistentLoop<KV8>::waves;
+    auto kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KV8, PW, PersistentLoop<KV8>::occ,
+                                                    Pipeline<KV8>::tiles_per_chunk>;
+    int resident = 0;
+    FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
+    const dim3 grid((unsigned)std::min<int64_t>(resident, items));
+    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
+  } else {
+    const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+    FA_HIP_CHECK(timer.launch(
+        paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ,
+                          (FA_LPT != 0), Pipeline<KV8>::tiles_per_chunk>,
+        grid, dim3(NW * 64), 0, p));
+  }
   if (r.elapsed_us) FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
   return FA_OK;
 }

@@ -34,7 +34,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
     auto kernel = paged_attn_split_persistent_kernel<HEAD_SIZE, QT, KV8, Pipeline<KV8>::occ,
                                                      Pipeline<KV8>::tiles_per_chunk>;
     int resident = 0;
-    FA_HIP_CHECK(resident_wavefronts(kernel, &resident));
+    FA_HIP_CHECK(resident_groups(kernel, 64, &resident));
     const int64_t max_items =
         (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
     const dim3 grid((unsigned)std::min<int64_t>(resident, max_items));

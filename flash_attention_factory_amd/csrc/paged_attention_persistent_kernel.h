@@ -23,7 +23,7 @@ constexpr int kPersistentMaxSeqs = 256;
 template <int D, typename QT, bool KV8, int OCC, int TPC>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_split_persistent_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KV8, TPC>;
+  using W = WaveAttn<D, QT, KV8, TPC, Pipeline<KV8>::stream_loads_split>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;

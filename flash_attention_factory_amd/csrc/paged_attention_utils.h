@@ -138,42 +138,38 @@ __device__ __forceinline__ int32_t load_uniform_i32(const int32_t *p) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// K/V bytes are read exactly once per launch: FA_STREAM_LOADS marks those loads
-// non-temporal so they do not displace the few lines that are re-used (queries, block
-// tables, the split path's scratch).
-#ifndef FA_STREAM_LOADS
-#define FA_STREAM_LOADS 0
-#endif
-template <typename T>
-__device__ __forceinline__ T stream_load(const T *p) {
-#if FA_STREAM_LOADS
-  return __builtin_nontemporal_load(p);
-#else
-  return *p;
-#endif
+// K/V bytes are read exactly once per launch.  STREAM marks a load non-temporal so that it
+// does not displace the few lines that are re-used (queries, block tables, scratch).
+template <bool STREAM, typename T>
+__device__ __forceinline__ T kv_load(const T *p) {
+  if constexpr (STREAM) {
+    return __builtin_nontemporal_load(p);
+  } else {
+    return *p;
+  }
 }
 
 // Global loads of 4, 8 or 16 bytes per lane.
-template <int DWORDS>
+template <int DWORDS, bool STREAM>
 struct VLoad;
-template <>
-struct VLoad<4> {
+template <bool STREAM>
+struct VLoad<4, STREAM> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[4], const char *p) {
-    u32x4 t = stream_load(reinterpret_cast<const u32x4 *>(p));
+    u32x4 t = kv_load<STREAM>(reinterpret_cast<const u32x4 *>(p));
     dst[0] = t[0]; dst[1] = t[1]; dst[2] = t[2]; dst[3] = t[3];
   }
 };
-template <>
-struct VLoad<2> {
+template <bool STREAM>
+struct VLoad<2, STREAM> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[2], const char *p) {
-    u32x2 t = stream_load(reinterpret_cast<const u32x2 *>(p));
+    u32x2 t = kv_load<STREAM>(reinterpret_cast<const u32x2 *>(p));
     dst[0] = t[0]; dst[1] = t[1];
   }
 };
-template <>
-struct VLoad<1> {
+template <bool STREAM>
+struct VLoad<1, STREAM> {
   static __device__ __forceinline__ void ld(uint32_t (&dst)[1], const char *p) {
-    dst[0] = stream_load(reinterpret_cast<const uint32_t *>(p));
+    dst[0] = kv_load<STREAM>(reinterpret_cast<const uint32_t *>(p));
   }
 };
 

@@ -22,10 +22,6 @@
 #include "paged_attention_policy.h"
 #include "paged_attention_utils.h"
 
-#ifndef FA_STREAM_STORES
-#define FA_STREAM_STORES 0
-#endif
-
 namespace fa {
 
 struct PagedAttnParams {
@@ -56,7 +52,7 @@ struct PagedAttnParams {
 
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
-template <int D, typename QT, bool KV8, int TPC>
+template <int D, typename QT, bool KV8, int TPC, bool STREAM>
 struct WaveAttn {
   static_assert(TPC == 2 || TPC == 4, "a chunk is one or two 32-token P.V steps");
   static constexpr int ROWB = D * (KV8 ? 1 : 2);  // bytes per token row
@@ -68,6 +64,7 @@ struct WaveAttn {
   static constexpr int CT = TPC * kTileTokens;    // tokens per chunk
   static constexpr int NP2 = TPC / 2;             // 32-token P.V steps per chunk
   static constexpr int NR = NDT * 4;              // accumulator values per lane
+  static constexpr bool kStream = STREAM;  // non-temporal K/V loads
 
   // Register image of one chunk of K and V.
   struct Chunk {
@@ -159,7 +156,7 @@ struct WaveAttn {
     for (int t = 0; t < TPC; ++t) {
       const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
 #pragma unroll
-      for (int c = 0; c < KL; ++c) R.k[t][c] = stream_load(reinterpret_cast<const u32x4 *>(kp + c * 64));
+      for (int c = 0; c < KL; ++c) R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + c * 64));
     }
   }
   __device__ __forceinline__ void issue_v(Chunk &R, int kvh, int ci, const Ids &ids) const {
@@ -168,7 +165,7 @@ struct WaveAttn {
       const char *vp = p.value_cache + tile_offset(kvh, ci, t, ids) +
                        (int64_t)(4 * r) * p.kv_token_bytes + i * VB;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) VLoad<VW>::ld(R.v[t * 4 + e], vp + e * p.kv_token_bytes);
+      for (int e = 0; e < 4; ++e) VLoad<VW, kStream>::ld(R.v[t * 4 + e], vp + e * p.kv_token_bytes);
     }
   }
 
@@ -290,11 +287,7 @@ struct WaveAttn {
 #pragma unroll
       for (int k = 0; k < N; k += 4) {
         f32x4 v = {o[k] * inv, o[k + 1] * inv, o[k + 2] * inv, o[k + 3] * inv};
-#if FA_STREAM_STORES
-        __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst + k));
-#else
         *reinterpret_cast<f32x4 *>(dst + k) = v;
-#endif
       }
     } else {
 #pragma unroll
