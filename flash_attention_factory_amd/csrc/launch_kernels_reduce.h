@@ -32,7 +32,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // length return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
   if (kUsePersistentSplit && shape.num_seqs <= kPersistentMaxSeqs && shape.num_pool_blocks > 0) {
     auto kernel = paged_attn_split_persistent_kernel<HEAD_SIZE, QT, KV8, Pipeline<KV8>::occ,
-                                                     Pipeline<KV8>::tiles_per_chunk>;
+                                                     Pipeline<KV8>::tiles_per_chunk, SplitOrder<KV8>::value>;
     int resident = 0;
     FA_HIP_CHECK(resident_groups(kernel, 64, &resident));
     const int64_t max_items =
@@ -58,8 +58,12 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   rp.max_num_partitions = shape.max_num_partitions;
   rp.partition_size = r.partition_size;
   rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
-  FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT>,
-                            dim3(shape.num_heads, shape.num_seqs), dim3(kReduceThreads), 1, rp));
+  const dim3 rgrid(shape.num_heads, shape.num_seqs);
+  if ((int64_t)shape.num_heads * shape.num_seqs >= kReduceSingleWaveMinPairs) {
+    FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1>, rgrid, dim3(64), 1, rp));
+  } else {
+    FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4>, rgrid, dim3(256), 1, rp));
+  }
   if (r.elapsed_us) {
     FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
     FA_HIP_CHECK(timer.read(1, &r.elapsed_us[1]));

@@ -20,7 +20,7 @@ namespace fa {
 
 constexpr int kPersistentMaxSeqs = 256;
 
-template <int D, typename QT, bool KV8, int OCC, int TPC>
+template <int D, typename QT, bool KV8, int OCC, int TPC, int ORDER>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_split_persistent_kernel(const PagedAttnParams p) {
   using W = WaveAttn<D, QT, KV8, TPC, Pipeline<KV8>::stream_loads_split>;
@@ -64,17 +64,21 @@ paged_attn_split_persistent_kernel(const PagedAttnParams p) {
   }
   const int total_items = running * Hk;
 
-  // item k -> (kv head, sequence, partition): kv head fastest, then partition, then sequence
+  // item k -> (sequence, kv head, partition).
+  //   ORDER 0: kv head fastest, then partition, then sequence.
+  //   ORDER 1: partition fastest, then kv head, then sequence -- neighbouring items write
+  //            neighbouring tmp_out rows (the partitions of one head are contiguous there).
   struct Item { int seq, kvh, part, tok_end, c_begin, c_end; };
   auto decode = [&](int k) -> Item {
     Item it;
     // integer division runs on the vector unit: tell the compiler the results are uniform
-    const int q = __builtin_amdgcn_readfirstlane(k / Hk);
-    it.kvh = k - q * Hk;
+    const int q = ORDER == 0 ? __builtin_amdgcn_readfirstlane(k / Hk) : k;
     int s = 0;
 #pragma unroll
     for (int j = 0; j < NQ; ++j)
-      if (j * 64 < S) s += __builtin_popcountll(__ballot(lane + 64 * j < S && incl[j] <= q));
+      if (j * 64 < S)
+        s += __builtin_popcountll(
+            __ballot(lane + 64 * j < S && (ORDER == 0 ? incl[j] : incl[j] * Hk) <= q));
     s = min(s, S - 1);
     int inc_s = 0, cnt_s = 0, ctx_s = 0;
 #pragma unroll
@@ -85,7 +89,14 @@ paged_attn_split_persistent_kernel(const PagedAttnParams p) {
         ctx_s = __builtin_amdgcn_readlane(ctxv[j], s & 63);
       }
     it.seq = __builtin_amdgcn_readfirstlane(s);
-    it.part = q - (inc_s - cnt_s);
+    if constexpr (ORDER == 0) {
+      it.kvh = k - q * Hk;
+      it.part = q - (inc_s - cnt_s);
+    } else {
+      const int rem = k - (inc_s - cnt_s) * Hk;
+      it.kvh = __builtin_amdgcn_readfirstlane(rem / max(cnt_s, 1));
+      it.part = rem - it.kvh * cnt_s;
+    }
     const int tok_begin = it.part * p.partition_size;
     it.tok_end = min(ctx_s, tok_begin + p.partition_size);
     it.c_begin = tok_begin / CT;
@@ -93,8 +104,22 @@ paged_attn_split_persistent_kernel(const PagedAttnParams p) {
     return it;
   };
 
-  int k = blockIdx.x;
-  if (k >= total_items) return;
+  // Which items this work-group walks: k_first, k_first + k_stride, ... below k_end.
+  //   ORDER 0: all work-groups interleave over the whole list.
+  //   ORDER 1: work-groups land on the 8 XCDs round-robin (id mod 8), each XCD with its own
+  //            L2; give every XCD one contiguous eighth of the list, interleaved among its
+  //            own work-groups, so rows that are neighbours in memory meet in one L2.
+  int k_first = blockIdx.x, k_stride = gridDim.x, k_end = total_items;
+  if constexpr (ORDER == 1) {
+    const int xcd = blockIdx.x & 7;
+    const int per_xcd = (total_items + 7) / 8;
+    k_stride = ((int)gridDim.x + 7 - xcd) / 8;
+    k_first = xcd * per_xcd + ((int)blockIdx.x >> 3);
+    k_end = min(total_items, (xcd + 1) * per_xcd);
+  }
+
+  int k = k_first;
+  if (k >= k_end) return;
 
   W wa(p, lane);
   const int col_max = p.max_blocks_per_seq - 1;  // ids are clamped into the pool or the
@@ -117,8 +142,8 @@ paged_attn_split_persistent_kernel(const PagedAttnParams p) {
       nk = kk;
       return true;
     }
-    nk = kk + gridDim.x;
-    if (nk >= total_items) return false;
+    nk = kk + k_stride;
+    if (nk >= k_end) return false;
     nit = decode(nk);
     nc = nit.c_begin;
     return true;

@@ -6,12 +6,12 @@
 //   out = sum_p (w_p / sum_q w_q) * tmp_out[p, :]      (compute_out :771-864, collect_out :868-934)
 // Only the ceil(context_len / partition_size) live partitions are read (:679,716).
 //
-// One work-group of four wavefronts per (sequence, head).  The kernel is a chain of
-// dependent memory round trips, so it is built to have as few of them as possible:
-// wavefront w owns partitions w, w+4, w+8, ... and requests up to 16 of their tmp_out
+// One work-group of one or four wavefronts per (sequence, head).  The kernel is a chain
+// of dependent memory round trips, so it is built to have as few of them as possible:
+// wavefront w owns partitions w, w+NW, w+2NW, ... and requests up to 16 of their tmp_out
 // rows (one coalesced 512-byte row per load) together with the partition scalars, before
-// anything is waited for; the weights are applied when both have arrived; the four
-// partial sums meet in LDS.  Lane j owns D/64 consecutive output elements.
+// anything is waited for; the weights are applied when both have arrived; with four
+// wavefronts the partial sums meet in LDS.  Lane j owns D/64 consecutive output elements.
 #pragma once
 
 #include "paged_attention_utils.h"
@@ -30,10 +30,13 @@ struct ReduceParams {
   int32_t max_context;  // max_blocks_per_seq * block_size: lengths are cut to it
 };
 
-constexpr int kReduceWaves = 4;
-constexpr int kReduceRowsInFlight = 16;  // per wavefront; 4 x 16 = 64 partitions per batch
+constexpr int kReduceRowsInFlight = 16;  // per wavefront and batch
 
-template <int D, typename QT>
+// kReduceWaves wavefronts per (sequence, head): 4 when there are few (sequence, head)
+// pairs -- the launch is then short of parallelism and each pair's rows should be in
+// flight at once -- 1 when there are thousands and every wavefront slot of the GPU is
+// filled anyway (no LDS, no barrier, more groups resident).
+template <int D, typename QT, int kReduceWaves>
 __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
   constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
   constexpr int R = kReduceRowsInFlight;
@@ -97,19 +100,24 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   }
   W = wave_sum(W);
 
-  __shared__ float part[kReduceWaves][D];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) part[wave][lane * EPL + e] = acc[e];
-  __syncthreads();
-  if (wave != 0) return;
   const float inv = 1.0f / W;
   float o[EPL];
+  if constexpr (kReduceWaves == 1) {
 #pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    float a = 0.f;
+    for (int e = 0; e < EPL; ++e) o[e] = acc[e] * inv;
+  } else {
+    __shared__ float part[kReduceWaves][D];
 #pragma unroll
-    for (int w = 0; w < kReduceWaves; ++w) a += part[w][lane * EPL + e];
-    o[e] = a * inv;
+    for (int e = 0; e < EPL; ++e) part[wave][lane * EPL + e] = acc[e];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      float a = 0.f;
+#pragma unroll
+      for (int w = 0; w < kReduceWaves; ++w) a += part[w][lane * EPL + e];
+      o[e] = a * inv;
+    }
   }
   char *dst = reinterpret_cast<char *>(p.out) +
               (((int64_t)seq * p.num_heads + head) * D + lane * EPL) * 2;

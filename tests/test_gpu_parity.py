@@ -176,6 +176,17 @@ def test_persistent_split_many_items_per_wavefront(oracle):
     torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("batch,heads", [(300, 16), (128, 32)])
+def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
+    """From 4096 (sequence, head) pairs on the reduce kernel runs one wavefront per pair;
+    lengths up to 9 partitions of 256 tokens exercise its multi-row batches."""
+    w = W.make_test_shaped(batch_size=batch, nheads=heads, nheads_k=2, d=64, seqlen_k=2300 if batch == 128 else 600,
+                           varlen=True, has_sinks=True, seed=batch)
+    assert w.num_seqs * w.num_heads >= 4096
+    bufs, _ = _run(w, "reduce")
+    _check(bufs.out, w, oracle, f"reduce 1-wave form, {batch} sequences x {heads} heads")
+
+
 def test_bf16_and_fp8_scale(oracle):
     # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
     w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,
