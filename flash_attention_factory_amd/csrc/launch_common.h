@@ -161,23 +161,30 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
 }
 
 // How many work-groups of `threads` threads of a kernel the current device keeps resident
-// (compute units x work-groups per compute unit).  Asked once per kernel and device.
-template <typename K>
-inline hipError_t resident_groups(K kernel, int threads, int *out) {
-  static thread_local int cached_dev = -1, cached = 0;
+// (compute units x work-groups per compute unit).  Asked once per (kernel, device); all
+// kernels here share one function-pointer type, so the cache is keyed by the pointer value.
+inline hipError_t resident_groups(void (*kernel)(PagedAttnParams), int threads, int *out) {
+  struct Entry { const void *fn; int dev; int groups; };
+  constexpr int kSlots = 64;
+  static thread_local Entry cache[kSlots];
+  static thread_local int used = 0;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev != cached_dev) {
-    int cus = 0, per_cu = 0;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
-    if (e != hipSuccess) return e;
-    cached = cus * (per_cu > 0 ? per_cu : 1);
-    cached_dev = dev;
-  }
-  *out = cached;
+  const void *fn = reinterpret_cast<const void *>(kernel);
+  for (int k = 0; k < used; ++k)
+    if (cache[k].fn == fn && cache[k].dev == dev) {
+      *out = cache[k].groups;
+      return hipSuccess;
+    }
+  int cus = 0, per_cu = 0;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return e;
+  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
+  if (e != hipSuccess) return e;
+  const int groups = cus * (per_cu > 0 ? per_cu : 1);
+  if (used < kSlots) cache[used++] = Entry{fn, dev, groups};
+  *out = groups;
   return hipSuccess;
 }
 
