@@ -31,7 +31,11 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (summaries under profiles/); None where not yet measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE + WRITE_SIZE of paged_attn_loop_persistent_kernel<128, F16, kv16> per launch,
+    # profiles/paged_attn_kernels_bench_configs.md
+    "config1_loop": 661.09e6 + 0.26e6,
+}
 
 
 def _clones(w, torch):
