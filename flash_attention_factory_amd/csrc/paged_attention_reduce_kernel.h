@@ -53,49 +53,45 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   const float *es = p.exp_sums + base;
   const float *tmp = p.tmp_out + base * D + lane * EPL;
 
-  // first batch of rows and the scalars go out together
+  // Partitions are handled in groups of 64 (lane q of the wavefront holds the weight of
+  // partition 64g + q); inside a group the rows go out in batches of R per wavefront.
+  // The first batch of rows and the scalars are requested together, before any wait.
+  constexpr int BATCH = kReduceWaves * R;  // rows per batch over the whole work-group
+  static_assert(64 % BATCH == 0, "a group of 64 partitions is a whole number of batches");
   float v[R][EPL];
-#pragma unroll
-  for (int u = 0; u < R; ++u) {
-    const int q = wave + kReduceWaves * u;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * D + e] : 0.f;
-  }
-  // lane q keeps the scalars of partition q (first 64 partitions) in registers
-  const float ml0 = (lane < np) ? ml[lane] : -INFINITY;
-  const float es0 = (lane < np) ? es[lane] : 0.f;
-  float M = ml0;
-  for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q]);
-  M = wave_max(M);
-  float w_lane = es0 * __expf(ml0 - M);  // weight of partition `lane`
-  float W = w_lane;
-
-  float acc[EPL];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
-#pragma unroll
-  for (int u = 0; u < R; ++u) {
-    const int q = wave + kReduceWaves * u;  // wave-uniform, < 64
-    const float w = __shfl(w_lane, q);      // 0 for q >= np
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
-  }
-  // contexts beyond 64 partitions: further batches of 64 partitions
-  for (int q0 = kReduceWaves * R; q0 < np; q0 += kReduceWaves * R) {
+  auto request_rows = [&](int q0) {
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int q = q0 + wave + kReduceWaves * u;
 #pragma unroll
       for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * D + e] : 0.f;
     }
-    const int ql = q0 + lane;
-    w_lane = (ql < np) ? es[ql] * __expf(ml[ql] - M) : 0.f;
+  };
+  request_rows(0);
+  // lane q keeps the scalars of partition q (first group) in registers
+  const float ml0 = (lane < np) ? ml[lane] : -INFINITY;
+  const float es0 = (lane < np) ? es[lane] : 0.f;
+  float M = ml0;
+  for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q]);
+  M = wave_max(M);
+
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+  float W = 0.f;
+  for (int g0 = 0; g0 < np; g0 += 64) {
+    const int ql = g0 + lane;
+    const float w_lane = g0 == 0 ? es0 * __expf(ml0 - M)
+                                 : ((ql < np) ? es[ql] * __expf(ml[ql] - M) : 0.f);
     W += w_lane;
+    for (int b0 = 0; b0 < 64 && g0 + b0 < np; b0 += BATCH) {
+      if (g0 + b0 > 0) request_rows(g0 + b0);
 #pragma unroll
-    for (int u = 0; u < R; ++u) {
-      const float w = __shfl(w_lane, wave + kReduceWaves * u);
+      for (int u = 0; u < R; ++u) {
+        const float w = __shfl(w_lane, b0 + wave + kReduceWaves * u);  // 0 past the last partition
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
+        for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
+      }
     }
   }
   W = wave_sum(W);

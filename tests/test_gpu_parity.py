@@ -180,11 +180,70 @@ def test_persistent_split_many_items_per_wavefront(oracle):
 def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
     """From 4096 (sequence, head) pairs on the reduce kernel runs one wavefront per pair;
     lengths up to 9 partitions of 256 tokens exercise its multi-row batches."""
-    w = W.make_test_shaped(batch_size=batch, nheads=heads, nheads_k=2, d=64, seqlen_k=2300 if batch == 128 else 600,
+    w = W.make_test_shaped(batch_size=batch, nheads=heads, nheads_k=2, d=64, seqlen_k=4500 if batch == 128 else 600,
                            varlen=True, has_sinks=True, seed=batch)
     assert w.num_seqs * w.num_heads >= 4096
+    if batch == 128:  # from 1 to more than 64 partitions per sequence: several row batches and groups
+        w.partition_size = 64
+        assert w.max_num_partitions > 64
+        w.context_lens[::3] = 4500 - torch.arange(0, 43, dtype=torch.int32) * 104
     bufs, _ = _run(w, "reduce")
     _check(bufs.out, w, oracle, f"reduce 1-wave form, {batch} sequences x {heads} heads")
+
+
+@pytest.mark.parametrize("index", [1, 2, 3, 4])
+def test_full_size_configs(oracle, index):
+    """The measured configurations at their full sizes.  The pools are drawn on the GPU
+    (a gigabyte of normals takes the host a minute) and copied back for the oracle, so
+    both sides see the same bytes.  Also checked at full size: loop == split + reduce,
+    and invariance under a permutation of the pool's blocks together with the tables."""
+    from flash_attention_factory_amd import runner
+    dev = _dev()
+    wd = W.make_config(index, device=dev, pools_on_device=True)
+    w = wd.to("cpu")
+    kernel = W.CONFIG_KERNEL[index]
+    bufs = runner.alloc_buffers(wd)
+    runner.run_workload(wd, kernel, bufs)
+    torch.cuda.synchronize()
+    _check(bufs.out, w, oracle, f"full {w.name}")
+    other = {"loop": "reduce", "reduce": "loop", "fp8_loop": "fp8_reduce", "fp8_reduce": "fp8_loop"}[kernel]
+    bufs2 = runner.alloc_buffers(wd)
+    runner.run_workload(wd, other, bufs2)
+    torch.cuda.synchronize()
+    a, b = bufs.out.float(), bufs2.out.float()
+    ulps = 2.0 ** (-7 if w.query.dtype == torch.bfloat16 else -10)  # two 16-bit roundings apart
+    assert (a - b).abs().max().item() <= ulps * a.abs().max().item() + 1e-5
+    # permute the pool's blocks and rewrite the tables: same answer, bit for bit
+    NB = wd.key_cache.shape[0]
+    perm = torch.randperm(NB, device=dev)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(NB, device=dev)
+    del bufs2
+    w2 = W.Workload(**{**wd.__dict__})
+    w2.key_cache = wd.key_cache[perm]
+    w2.value_cache = wd.value_cache[perm]
+    w2.block_tables = inv[wd.block_tables.long()].to(torch.int32)
+    bufs3 = runner.alloc_buffers(w2)
+    runner.run_workload(w2, kernel, bufs3)
+    torch.cuda.synchronize()
+    assert torch.equal(bufs3.out, bufs.out)
+
+
+def test_persistent_kernels_small_batches(oracle):
+    """Fewer items than resident work-groups, a single sequence, a batch where most
+    wavefronts of a loop work-group have no chunk, and 128 sequences (the limit of the
+    persistent loop kernel) next to 129 (grid form)."""
+    cases = [
+        W.make_config(1, num_seqs=1, pool_blocks=200, lens=[1999]),
+        W.make_config(0, num_seqs=3, pool_blocks=64, lens=[5, 40, 33]),
+        W.make_config(3, num_seqs=2, pool_blocks=300, lens=[17, 2048]),
+        W.make_config(0, num_seqs=128, pool_blocks=128 * 8, lens=[(7 * s) % 120 + 1 for s in range(128)]),
+        W.make_config(0, num_seqs=129, pool_blocks=129 * 8, lens=[(11 * s) % 120 + 1 for s in range(129)]),
+    ]
+    for w in cases:
+        for kernel in (("fp8_loop", "fp8_reduce") if w.is_fp8 else ("loop", "reduce")):
+            bufs, _ = _run(w, kernel)
+            _check(bufs.out, w, oracle, f"{w.name} S={w.num_seqs}/{kernel}")
 
 
 def test_bf16_and_fp8_scale(oracle):
