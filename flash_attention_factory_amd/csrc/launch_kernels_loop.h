@@ -39,8 +39,8 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   } else {
     const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ,
-                          (FA_LPT != 0), Pipeline<KV8>::tiles_per_chunk>,
+        paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::occ,
+                          Pipeline<KV8>::tiles_per_chunk>,
         grid, dim3(NW * 64), 0, p));
   }
   if (r.elapsed_us) FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));

@@ -42,8 +42,8 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   } else {
     const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::pipe, Pipeline<KV8>::occ,
-                          false, Pipeline<KV8>::tiles_per_chunk>,
+        paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::occ,
+                          Pipeline<KV8>::tiles_per_chunk>,
         grid, dim3(NW * 64), 0, p));
   }
 

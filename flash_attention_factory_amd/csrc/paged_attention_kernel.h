@@ -89,7 +89,7 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   }
 }
 
-template <int D, typename QT, bool KV8, bool PART, int NW, int PIPE, int OCC, bool LPT, int TPC>
+template <int D, typename QT, bool KV8, bool PART, int NW, int OCC, int TPC>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {
   using W = WaveAttn<D, QT, KV8, TPC, PART ? Pipeline<KV8>::stream_loads_split : Pipeline<KV8>::stream_loads_loop>;
@@ -101,29 +101,7 @@ paged_attn_kernel(const PagedAttnParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.x;
   const int part = blockIdx.y;
-  // Which sequence this work-group takes.  Work-groups are dispatched in blockIdx
-  // order (z slowest); handing the longest sequences to the lowest z means the tail of
-  // the launch is made of the shortest ones.  Every wavefront ranks the context lengths
-  // by itself (no LDS, no barrier); done for up to 128 sequences, identity beyond.
-  int seq = blockIdx.z;
-  if constexpr (LPT) {
-    const int S = gridDim.z;
-    if (S > 1 && S <= 128) {
-      const int len0 = lane < S ? p.context_lens[lane] : -1;
-      const int len1 = lane + 64 < S ? p.context_lens[lane + 64] : -1;
-      int rank0 = 0, rank1 = 0;
-      for (int u = 0; u < S; ++u) {
-        const int lu = u < 64 ? __builtin_amdgcn_readlane(len0, u)
-                              : __builtin_amdgcn_readlane(len1, u - 64);
-        rank0 += (lu > len0) || (lu == len0 && u < lane);
-        rank1 += (lu > len1) || (lu == len1 && u < lane + 64);
-      }
-      const unsigned long long b0 = __ballot(lane < S && rank0 == (int)blockIdx.z);
-      const unsigned long long b1 = __ballot(lane + 64 < S && rank1 == (int)blockIdx.z);
-      seq = b0 ? __builtin_ctzll(b0) : 64 + __builtin_ctzll(b1);
-      seq = __builtin_amdgcn_readfirstlane(seq);
-    }
-  }
+  const int seq = blockIdx.z;
 
   W wa(p, lane);
   const int tok_begin = PART ? part * p.partition_size : 0;
@@ -156,55 +134,27 @@ paged_attn_kernel(const PagedAttnParams p) {
   int ci = c_begin + wave;
   if (ci < c_end) {
     if (!pool_known) ids0 = wa.fetch_ids(table, ci, last_blk);
-    if constexpr (PIPE == 1) {
-      // One register set.  K of chunk n+1 is requested as soon as the score MFMAs of
-      // chunk n have read K, V of chunk n+1 as soon as the P.V MFMAs have read V: about
-      // half a chunk is in flight per wavefront at any time, at half the registers.
-      Chunk R;
-      wa.issue_k(R, kvh, ci, ids0);
-      wa.issue_v(R, kvh, ci, ids0);
-      Ids nids = wa.fetch_ids(table, ci + NW, last_blk);
-      while (ci + NW < c_end) {
-        const int cn = ci + NW;
-        const auto s = wa.qk(R);
-        wa.issue_k(R, kvh, cn, nids);
-        const auto pb = wa.template soft<false>(R, s, ci, tok_end);
-        wa.pv(R, pb);
-        wa.issue_v(R, kvh, cn, nids);
-        nids = wa.fetch_ids(table, cn + NW, last_blk);
-        ci = cn;
-      }
+    // One register set.  K of chunk n+1 is requested as soon as the score MFMAs of
+    // chunk n have read K, V of chunk n+1 as soon as the P.V MFMAs have read V: about
+    // half a chunk is in flight per wavefront at any time.  (Two register sets with the
+    // whole next chunk in flight were measured too: same bandwidth, a third fewer
+    // wavefronts resident.)
+    Chunk R;
+    wa.issue_k(R, kvh, ci, ids0);
+    wa.issue_v(R, kvh, ci, ids0);
+    Ids nids = wa.fetch_ids(table, ci + NW, last_blk);
+    while (ci + NW < c_end) {
+      const int cn = ci + NW;
       const auto s = wa.qk(R);
-      wa.pv(R, wa.template soft<true>(R, s, ci, tok_end));
-    } else {
-      // Two register sets: all loads of chunk n+1 are in flight under chunk n.
-      Chunk A, B;
-      wa.issue_k(A, kvh, ci, ids0);
-      wa.issue_v(A, kvh, ci, ids0);
-      Ids nids = wa.fetch_ids(table, ci + NW, last_blk);
-      while (true) {
-        int cn = ci + NW;
-        if (cn >= c_end) {
-          wa.pv(A, wa.template soft<true>(A, wa.qk(A), ci, tok_end));
-          break;
-        }
-        wa.issue_k(B, kvh, cn, nids);
-        wa.issue_v(B, kvh, cn, nids);
-        nids = wa.fetch_ids(table, cn + NW, last_blk);
-        wa.pv(A, wa.template soft<false>(A, wa.qk(A), ci, tok_end));
-        ci = cn;
-        cn = ci + NW;
-        if (cn >= c_end) {
-          wa.pv(B, wa.template soft<true>(B, wa.qk(B), ci, tok_end));
-          break;
-        }
-        wa.issue_k(A, kvh, cn, nids);
-        wa.issue_v(A, kvh, cn, nids);
-        nids = wa.fetch_ids(table, cn + NW, last_blk);
-        wa.pv(B, wa.template soft<false>(B, wa.qk(B), ci, tok_end));
-        ci = cn;
-      }
+      wa.issue_k(R, kvh, cn, nids);
+      const auto pb = wa.template soft<false>(R, s, ci, tok_end);
+      wa.pv(R, pb);
+      wa.issue_v(R, kvh, cn, nids);
+      nids = wa.fetch_ids(table, cn + NW, last_blk);
+      ci = cn;
     }
+    const auto s = wa.qk(R);
+    wa.pv(R, wa.template soft<true>(R, s, ci, tok_end));
   }
 
   merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part);

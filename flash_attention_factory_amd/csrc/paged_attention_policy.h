@@ -1,6 +1,8 @@
 // Compile-time tuning constants of the gfx950 kernels.  Plays the role of the
 // upstream policy header (include/paged_attention_policy_v2.hpp:5-100), but the
 // knobs are those of a wavefront-streaming design, not of sub-group tiling.
+// Every default below is the measured best on MI355X; each can be overridden with -D
+// for experiments.
 #pragma once
 
 namespace fa {
@@ -18,9 +20,10 @@ constexpr int default_partition_size(int head_size) { return head_size == 64 ? 2
 // Query heads sharing one kv head are packed as the 16 columns of an MFMA tile.
 constexpr int kMaxGroup = 16;
 
+// ---- grid-form kernels (any batch size) ----------------------------------------------
 // Wavefronts per work-group.
 //  * loop kernel: one work-group owns a whole (sequence, kv head); its wavefronts
-//    interleave 32-token chunks and merge once at the end through LDS.
+//    interleave chunks and merge once at the end through LDS.
 //  * split kernel: one work-group owns one partition of one (sequence, kv head).
 #ifndef FA_LOOP_WAVES
 #define FA_LOOP_WAVES 8
@@ -33,18 +36,12 @@ struct WavesPerGroup {
   static constexpr int value = kPartitioned ? FA_SPLIT_WAVES : FA_LOOP_WAVES;
 };
 
-// Streaming pipeline of the attention kernel and the occupancy it is compiled for.
-//   PIPE 0: two register sets, the whole next chunk in flight under the current one.
-//   PIPE 1: one register set, K and V refilled separately right after their MFMAs.
-//   OCC   : wavefronts per SIMD the register allocator must fit (4 SIMDs per CU).
-#ifndef FA_PIPE
-#define FA_PIPE 1
-#endif
+// Per cache type: wavefronts per SIMD the register allocator must fit (4 SIMDs per CU),
+// tiles per chunk, and whether K/V loads are marked non-temporal (the bytes are read once
+// per launch).  Non-temporal loads measured +4..5 % on 16-bit caches in both paths and
+// +10 % on the FP8 loop path, but -3 % on the FP8 split path.
 #ifndef FA_OCC
 #define FA_OCC 3
-#endif
-#ifndef FA_PIPE_FP8
-#define FA_PIPE_FP8 FA_PIPE
 #endif
 #ifndef FA_OCC_FP8
 #define FA_OCC_FP8 FA_OCC
@@ -55,8 +52,6 @@ struct WavesPerGroup {
 #ifndef FA_TPC_FP8
 #define FA_TPC_FP8 2
 #endif
-// Non-temporal K/V loads (the bytes are read once per launch).  Measured: +4..5 % on
-// 16-bit caches in both paths, +10 % on the FP8 loop path, -3 % on the FP8 split path.
 #ifndef FA_STREAM_LOADS
 #define FA_STREAM_LOADS 1
 #endif
@@ -68,14 +63,14 @@ struct WavesPerGroup {
 #endif
 template <bool kKV8>
 struct Pipeline {
-  static constexpr int pipe = kKV8 ? FA_PIPE_FP8 : FA_PIPE;
   static constexpr int occ = kKV8 ? FA_OCC_FP8 : FA_OCC;
   static constexpr int tiles_per_chunk = kKV8 ? FA_TPC_FP8 : FA_TPC;
   static constexpr bool stream_loads_loop = (kKV8 ? FA_STREAM_LOADS_FP8_LOOP : FA_STREAM_LOADS) != 0;
   static constexpr bool stream_loads_split = (kKV8 ? FA_STREAM_LOADS_FP8_SPLIT : FA_STREAM_LOADS) != 0;
 };
 
-// Split path: use the persistent attention kernel when the batch allows it.
+// ---- persistent kernels (batches of up to 128 / 256 sequences) -------------------------
+// Split path: resident single-wavefront work-groups walk the live partitions.
 #ifndef FA_PERSISTENT_SPLIT
 #define FA_PERSISTENT_SPLIT 1
 #endif
@@ -94,8 +89,7 @@ struct SplitOrder {
   static constexpr int value = kKV8 ? FA_SPLIT_ORDER_FP8 : FA_SPLIT_ORDER;
 };
 
-
-// Loop path: use the persistent kernel when the batch allows it.
+// Loop path: resident work-groups walk the (sequence, kv head) items, longest first.
 #ifndef FA_PERSISTENT_LOOP
 #define FA_PERSISTENT_LOOP 1
 #endif
@@ -120,12 +114,8 @@ struct PersistentLoop {
   static constexpr int occ = kKV8 ? FA_PLOOP_OCC_FP8 : FA_PLOOP_OCC;
 };
 
-// Longest-sequence-first assignment of sequences to work-groups (loop kernel).
-#ifndef FA_LPT
-#define FA_LPT 0
-#endif
-
-// Reduce kernel: one wavefront per (sequence, head) from this many pairs on, four below.
+// ---- reduce kernel ---------------------------------------------------------------------
+// One wavefront per (sequence, head) from this many pairs on, four below.
 #ifndef FA_REDUCE_1W_MIN_PAIRS
 #define FA_REDUCE_1W_MIN_PAIRS 4096
 #endif
