@@ -9,8 +9,11 @@
 // a list of items:
 //   * items are ordered longest first (every wavefront ranks context_lens in registers)
 //     and dealt to the work-groups in snake order, so the work-groups' totals are even;
-//   * before a wavefront enters the merge of an item it has already requested the query
-//     rows and the first K/V chunk of the next item, so its stream never drains.
+//   * a wavefront that is through with its chunks of an item has already requested the
+//     query rows and the first K/V chunk of the next item; it parks its softmax state in
+//     LDS and goes on.  The states of an item are merged one chunk later, when all
+//     wavefronts have as a rule long delivered theirs: there is no barrier between items
+//     and the stream never drains.
 // Built for up to 128 sequences; larger batches use the grid form.
 #pragma once
 
@@ -19,6 +22,10 @@
 namespace fa {
 
 constexpr int kLoopPersistentMaxSeqs = 128;
+// Upper bound on the polls of one wait for the other wavefronts of a work-group (each poll
+// sleeps ~64 cycles).  Never reached in a correct run -- every wavefront publishes every
+// item -- it only turns a would-be hang into a wrong answer that the tests catch.
+constexpr int kLoopPersistentSpinLimit = 1 << 24;
 
 template <int D, typename QT, bool KV8, int NW, int OCC, int TPC>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
@@ -69,9 +76,11 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
   };
 
-  __shared__ float sm_m[NW][16];
-  __shared__ float sm_l[NW][16];
-  __shared__ float sm_acc[NW][NR][64];
+  // Partial states of two items in flight: item n goes to buffer n & 1.
+  __shared__ float sm_m[2][NW][16];
+  __shared__ float sm_l[2][NW][16];
+  __shared__ float sm_acc[2][NW][NR][64];
+  __shared__ int sm_arrived[2];  // wavefronts that have published into the buffer, ever
 
   W wa(p, lane);
   const int r = wa.r, i = wa.i;
@@ -79,7 +88,68 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
 
   int n = 0;
   Item cur;
-  if (!item_at(0, cur)) return;
+  if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
+  if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
+  __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
+
+  // A wavefront's state of item n goes to LDS and the wavefront moves on; nobody waits here.
+  auto publish = [&](int item) {
+    const int b = item & 1;
+    wa.l = rows_sum(wa.l);
+    if (r == 0) {
+      sm_m[b][wave][i] = wa.m;
+      sm_l[b][wave][i] = wa.l;
+    }
+#pragma unroll
+    for (int k = 0; k < NR; ++k) sm_acc[b][wave][k][lane] = wa.acc_at(k);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0)
+      __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  // Merge the NW published states of an item, normalise, store this wavefront's slice.
+  // Called one chunk into the following item (or after the last item), when the other
+  // wavefronts have as a rule long published: the wait below is then a single read.
+  // Every wavefront publishes every item in order, so the count is always reached; a
+  // wavefront calls finish(item) before it publishes item + 1, and finish(item) returns
+  // only after all have published `item`, hence after all have finished item - 1: a
+  // buffer is never overwritten while somebody still reads it.
+  auto finish = [&](int item, int seq, int kvh) {
+    const int b = item & 1;
+    const int target = NW * ((item >> 1) + 1);
+    for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
+      const int seen = __hip_atomic_load(&sm_arrived[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[b][w][i]);
+    float f[NW];
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float mw = sm_m[b][w][i];
+      f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
+      L += f[w] * sm_l[b][w][i];
+    }
+    float o[SL];
+#pragma unroll
+    for (int k = 0; k < SL; ++k) {
+      float a = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + k][lane];
+      o[k] = a;
+    }
+    if (i < p.group) {
+      const int head = kvh * p.group + i;
+      const int d0 = 4 * r * NDT + wave * SL;
+      W::template store_q<SL>(reinterpret_cast<char *>(p.out) +
+                                  (((int64_t)seq * p.num_heads + head) * D + d0) * 2,
+                              o, p.out_scale / L);
+    }
+  };
+
   // first chunk of the first item
   bool armed = wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
   if (armed) {
@@ -89,6 +159,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     wa.issue_v(R, cur.kvh, wave, ids);
   }
   uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0);
+  Item prev = cur;  // the item whose merge is still owed (from the second item on)
 
   while (true) {
     Item nxt;
@@ -100,19 +171,36 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
 
     wa.reset(sink_raw);
     uint32_t next_sink = W::kNoSink;
+    bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;
       int ci = wave;
       Ids nids = wa.fetch_ids(table, ci + NW, col_max);
-      while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
-        const int cn = ci + NW;
-        const auto s = wa.qk(R);
-        wa.issue_k(R, cur.kvh, cn, nids);
-        const auto pb = wa.template soft<false>(R, s, ci, cur.ctx);
-        wa.pv(R, pb);
-        wa.issue_v(R, cur.kvh, cn, nids);
-        nids = wa.fetch_ids(table, cn + NW, col_max);
-        ci = cn;
+      if (ci + NW < cur.c_end) {
+        {  // first chunk of the item, then the merge owed to the previous item
+          const int cn = ci + NW;
+          const auto s = wa.qk(R);
+          wa.issue_k(R, cur.kvh, cn, nids);
+          const auto pb = wa.template soft<false>(R, s, ci, cur.ctx);
+          wa.pv(R, pb);
+          wa.issue_v(R, cur.kvh, cn, nids);
+          nids = wa.fetch_ids(table, cn + NW, col_max);
+          ci = cn;
+        }
+        if (owed) {
+          finish(n - 1, prev.seq, prev.kvh);
+          owed = false;
+        }
+        while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
+          const int cn = ci + NW;
+          const auto s = wa.qk(R);
+          wa.issue_k(R, cur.kvh, cn, nids);
+          const auto pb = wa.template soft<false>(R, s, ci, cur.ctx);
+          wa.pv(R, pb);
+          wa.issue_v(R, cur.kvh, cn, nids);
+          nids = wa.fetch_ids(table, cn + NW, col_max);
+          ci = cn;
+        }
       }
       // last chunk of this wavefront in `cur`: what goes out next belongs to `nxt`
       const auto s = wa.qk(R);
@@ -130,50 +218,17 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       wa.issue_k(R, nxt.kvh, wave, nxt_ids);
       wa.issue_v(R, nxt.kvh, wave, nxt_ids);
     }
-
-    // ---- merge the NW wavefront states of `cur`, normalise, store ----------------------
-    wa.l = rows_sum(wa.l);
-    if (n > 0) __syncthreads();  // the previous item's partials have been read by everyone
-    if (r == 0) {
-      sm_m[wave][i] = wa.m;
-      sm_l[wave][i] = wa.l;
-    }
-#pragma unroll
-    for (int k = 0; k < NR; ++k) sm_acc[wave][k][lane] = wa.acc_at(k);
-    __syncthreads();
-    float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[w][i]);
-    float f[NW];
-    float L = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const float mw = sm_m[w][i];
-      f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
-      L += f[w] * sm_l[w][i];
-    }
-    float o[SL];
-#pragma unroll
-    for (int k = 0; k < SL; ++k) {
-      float a = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[w][wave * SL + k][lane];
-      o[k] = a;
-    }
-    if (i < p.group) {
-      const int head = cur.kvh * p.group + i;
-      const int d0 = 4 * r * NDT + wave * SL;
-      W::template store_q<SL>(reinterpret_cast<char *>(p.out) +
-                                  (((int64_t)cur.seq * p.num_heads + head) * D + d0) * 2,
-                              o, p.out_scale / L);
-    }
+    if (owed) finish(n - 1, prev.seq, prev.kvh);
+    publish(n);
 
     if (!has_next) break;
+    prev = cur;
     cur = nxt;
     armed = next_armed;
     sink_raw = next_sink;
     ++n;
   }
+  finish(n, cur.seq, cur.kvh);
 }
 
 }  // namespace fa
