@@ -26,7 +26,9 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
                                         block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
-  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0) {
+  const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
+  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
+      max_ctx < kLoopPersistentMaxContext) {
     // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
     // sequences first, with the next item's first loads issued before each merge.
     constexpr int PW = PersistentLoop<KV8>::waves;

@@ -14,7 +14,7 @@
 //     LDS and goes on.  The states of an item are merged one chunk later, when all
 //     wavefronts have as a rule long delivered theirs: there is no barrier between items
 //     and the stream never drains.
-// Built for up to 128 sequences; larger batches use the grid form.
+// Built for up to 128 sequences of fewer than 2^24 tokens; anything else uses the grid form.
 #pragma once
 
 #include "paged_attention_kernel.h"
@@ -22,6 +22,7 @@
 namespace fa {
 
 constexpr int kLoopPersistentMaxSeqs = 128;
+constexpr int kLoopPersistentMaxContext = 1 << 24;  // lengths are packed into 24 bits of a sort key
 // Upper bound on the polls of one wait for the other wavefronts of a work-group (each poll
 // sleeps ~64 cycles).  Never reached in a correct run -- every wavefront publishes every
 // item -- it only turns a would-be hang into a wrong answer that the tests catch.
@@ -50,16 +51,45 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   const int col_max = p.max_blocks_per_seq - 1;
 
   // ---- rank the sequences by length, longest first; lane holds sequences lane, lane+64 --
+  // Requested together with the lengths, so that the first K/V loads depend on one round
+  // trip to memory, not two: for EVERY sequence, the block ids of the chunk this wavefront
+  // would start with.  Once the ranking has named the first item its ids are a lane away.
   int len0 = -1, len1 = -1;
-  if (lane < S) len0 = max(0, min(p.context_lens[lane], max_ctx));
-  if (S > 64 && lane + 64 < S) len1 = max(0, min(p.context_lens[lane + 64], max_ctx));
-  int rank0 = 0, rank1 = 0;
-  for (int u = 0; u < S; ++u) {
-    const int lu = u < 64 ? __builtin_amdgcn_readlane(len0, u) : __builtin_amdgcn_readlane(len1, u - 64);
-    rank0 += (lu > len0) || (lu == len0 && u < lane);
-    rank1 += (lu > len1) || (lu == len1 && u < lane + 64);
+  int sid0[TPC] = {}, sid1[TPC] = {};
+  if (lane < S) {
+    len0 = max(0, min(p.context_lens[lane], max_ctx));
+    const int32_t *row = p.block_tables + (int64_t)lane * p.max_blocks_per_seq;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) sid0[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
   }
-
+  if (S > 64 && lane + 64 < S) {
+    len1 = max(0, min(p.context_lens[lane + 64], max_ctx));
+    const int32_t *row = p.block_tables + (int64_t)(lane + 64) * p.max_blocks_per_seq;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) sid1[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
+  }
+  // Sort key: length, then lower sequence number first; distinct for distinct sequences
+  // (lengths stay below 2^24, the launcher sees to that).  Lanes without a sequence: -1.
+  const int key0 = len0 < 0 ? -1 : (len0 << 7) | (127 - lane);
+  const int key1 = len1 < 0 ? -1 : (len1 << 7) | (63 - lane);
+  int rank0 = 0, rank1 = 0;  // how many sequences come before this one
+  // eight sequences per trip; lanes past the batch hold -1 and count for nothing
+  for (int u0 = 0; u0 < min(S, 64); u0 += 8) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int ku = __builtin_amdgcn_readlane(key0, u0 + j);
+      rank0 += ku > key0;
+      rank1 += ku > key1;
+    }
+  }
+  for (int u0 = 0; u0 < S - 64; u0 += 8) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int ku = __builtin_amdgcn_readlane(key1, u0 + j);
+      rank0 += ku > key0;
+      rank1 += ku > key1;
+    }
+  }
   struct Item { int seq, kvh, ctx, c_end; };
   // n-th item of this work-group: position n*G + j on even n, n*G + G-1-j on odd n
   auto item_at = [&](int n, Item &it) -> bool {
@@ -67,8 +97,8 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     if (pos >= T) return false;
     const int rho = __builtin_amdgcn_readfirstlane(pos / Hk);
     it.kvh = pos - rho * Hk;
-    const unsigned long long b0 = __ballot(lane < S && rank0 == rho);
-    const unsigned long long b1 = __ballot(lane + 64 < S && rank1 == rho);
+    const unsigned long long b0 = __ballot(key0 >= 0 && rank0 == rho);
+    const unsigned long long b1 = __ballot(key1 >= 0 && rank1 == rho);
     const int s = b0 ? __builtin_ctzll(b0) : 64 + __builtin_ctzll(b1);
     it.seq = __builtin_amdgcn_readfirstlane(s);
     it.ctx = s < 64 ? __builtin_amdgcn_readlane(len0, s) : __builtin_amdgcn_readlane(len1, s - 64);
@@ -153,7 +183,13 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   // first chunk of the first item
   bool armed = wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
   if (armed) {
-    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, wave, col_max);
+    Ids ids;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) {
+      const int raw = cur.seq < 64 ? __builtin_amdgcn_readlane(sid0[t], cur.seq)
+                                   : __builtin_amdgcn_readlane(sid1[t], cur.seq - 64);
+      ids.v[t] = min((uint32_t)raw, (uint32_t)p.max_block_id);
+    }
     wa.load_q(cur.seq, cur.kvh);
     wa.issue_k(R, cur.kvh, wave, ids);
     wa.issue_v(R, cur.kvh, wave, ids);

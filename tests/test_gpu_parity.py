@@ -246,6 +246,17 @@ def test_persistent_kernels_small_batches(oracle):
             _check(bufs.out, w, oracle, f"{w.name} S={w.num_seqs}/{kernel}")
 
 
+def test_table_wider_than_the_persistent_loop_key(oracle):
+    """A block table that could hold 2^24 tokens or more per sequence is outside what the
+    persistent loop kernel packs into its sort key; the launcher must take the grid form."""
+    w = W.make_config(0, num_seqs=2, pool_blocks=64, lens=[40, 33])
+    wide = torch.zeros((2, (1 << 24) // w.block_size), dtype=torch.int32)
+    wide[:, :w.block_tables.shape[1]] = w.block_tables
+    w.block_tables = wide
+    bufs, _ = _run(w, "loop")
+    _check(bufs.out, w, oracle, "2^24-token table/loop")
+
+
 def test_bf16_and_fp8_scale(oracle):
     # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
     w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,
