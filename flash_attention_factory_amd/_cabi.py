@@ -1,4 +1,5 @@
-"""ctypes binding of libfa_paged_attention.so (declarations: include/fa_paged_attention.h).
+"""ctypes binding of libfa_paged_attention.so (declarations: include/fa_paged_attention.h,
+include/fa_kv_cache.h).
 
 There is no fallback: if the HIP library is missing or a call fails, this raises.
 """
@@ -29,7 +30,11 @@ EXPORTS = (
     "fa_paged_attention_fp8_reduce",
     "fa_last_error",
     "fa_paged_attention_abi_version",
+    "fa_kv_cache_write",
 )
+
+FA_KV_CACHE_16BIT = 0
+FA_KV_CACHE_E5M2 = 1
 
 
 class Shape(ctypes.Structure):
@@ -63,6 +68,23 @@ class Options(ctypes.Structure):
     ]
 
 
+class KvWriteShape(ctypes.Structure):
+    _fields_ = [
+        ("num_tokens", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_size", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+        ("kv_block_stride", ctypes.c_int64),
+        ("kv_token_stride", ctypes.c_int64),
+        ("kv_head_stride", ctypes.c_int64),
+        ("src_token_stride", ctypes.c_int64),
+        ("src_head_stride", ctypes.c_int64),
+        ("src_dtype", ctypes.c_int32),
+        ("cache_dtype", ctypes.c_int32),
+        ("num_pool_blocks", ctypes.c_int64),
+    ]
+
+
 class PagedAttentionError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"[fa_status {code}] {message}")
@@ -93,6 +115,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(L, name)
         fn.argtypes = common + [P, P, P] + tail
         fn.restype = ctypes.c_int32
+    L.fa_kv_cache_write.argtypes = [P, P, P, P, P, ctypes.POINTER(KvWriteShape), ctypes.POINTER(Options)]
+    L.fa_kv_cache_write.restype = ctypes.c_int32
     L.fa_last_error.restype = ctypes.c_char_p
     L.fa_paged_attention_abi_version.restype = ctypes.c_int32
     _lib = L

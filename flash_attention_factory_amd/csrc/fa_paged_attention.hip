@@ -1,11 +1,14 @@
-// extern "C" surface of libfa_paged_attention.so: four entry points, one per host
-// launcher, declared in include/fa_paged_attention.h.
+// extern "C" surface of libfa_paged_attention.so: four decode entry points, one per host
+// launcher, declared in include/fa_paged_attention.h, and the KV-cache writer declared in
+// include/fa_kv_cache.h.
+#include "../../include/fa_kv_cache.h"
 #include "../../include/fa_paged_attention.h"
 
 #include "launch_kernels_fp8_loop.h"
 #include "launch_kernels_fp8_reduce.h"
 #include "launch_kernels_loop.h"
 #include "launch_kernels_reduce.h"
+#include "launch_kv_cache_write.h"
 
 #define FA_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -56,6 +59,13 @@ FA_EXPORT int32_t fa_paged_attention_fp8_reduce(void *out, const void *query,
                                           max_logits, tmp_out, shape, options);
 }
 
+FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *key_cache,
+                                    void *value_cache, const int64_t *slot_mapping,
+                                    const fa_kv_cache_write_shape *shape,
+                                    const fa_paged_attention_options *options) {
+  return fa::launch_kv_cache_write(key, value, key_cache, value_cache, slot_mapping, shape, options);
+}
+
 FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
 
-FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 1; }
+FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 2; }

@@ -41,6 +41,24 @@ class _Problem(ctypes.Structure):
     ]
 
 
+class _KvWrite(ctypes.Structure):
+    _fields_ = [
+        ("num_tokens", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_size", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+        ("kv_block_stride", ctypes.c_int64),
+        ("kv_token_stride", ctypes.c_int64),
+        ("kv_head_stride", ctypes.c_int64),
+        ("src_token_stride", ctypes.c_int64),
+        ("src_head_stride", ctypes.c_int64),
+        ("src_dtype", ctypes.c_int32),
+        ("cache_dtype", ctypes.c_int32),
+        ("num_pool_blocks", ctypes.c_int64),
+        ("fp8_scale", ctypes.c_float),
+    ]
+
+
 def build(force: bool = False) -> str:
     """Compile the C restatement with the Makefile next to it."""
     if force or not os.path.exists(_LIB_PATH):
@@ -75,6 +93,12 @@ def lib() -> ctypes.CDLL:
         L.oracle_e5m2_to_f32.argtypes = [ctypes.c_uint8]
         L.oracle_e5m2_to_f32.restype = ctypes.c_float
         L.oracle_num_threads.restype = ctypes.c_int
+        L.oracle_f32_to_e5m2.argtypes = [ctypes.c_float]
+        L.oracle_f32_to_e5m2.restype = ctypes.c_uint8
+        L.oracle_f32_to_e5m2_array.argtypes = [P, P, ctypes.c_int64]
+        L.oracle_f32_to_e5m2_array.restype = None
+        L.oracle_kv_cache_write.argtypes = [P, P, P, P, P, ctypes.POINTER(_KvWrite)]
+        L.oracle_kv_cache_write.restype = ctypes.c_int
         L.oracle_set_num_threads.argtypes = [ctypes.c_int]
         _lib = L
     return _lib
@@ -186,6 +210,39 @@ def kernel_reduce(exp_sums, max_logits, tmp_out, context_lens, *, partition_size
                                _ptr(tmp_out), _ptr(context_lens), partition_size, NP,
                                ctypes.byref(pr))
     return (out, out32) if want_f32 else out
+
+
+def f32_to_e5m2(values: torch.Tensor) -> torch.Tensor:
+    """Element-wise fp32 -> E5M2 byte (round to nearest even, overflow to infinity)."""
+    src = values.to(torch.float32).contiguous()
+    out = torch.empty(src.shape, dtype=torch.uint8)
+    lib().oracle_f32_to_e5m2_array(_ptr(src), _ptr(out), ctypes.c_int64(src.numel()))
+    return out
+
+
+def kv_cache_write(key, value, key_cache, value_cache, slot_mapping, *, block_size, kv_strides,
+                   fp8_scale=1.0):
+    """Scatter the rows of `key`/`value` ([N, Hk, D], fp16/bf16) into the paged pools in place
+    (the pool build of test_paged_fp8cache.py:171-203 as a per-token scatter)."""
+    assert key.device.type == "cpu" and key.dim() == 3 and key.stride(2) == 1
+    assert value.shape == key.shape and value.stride() == key.stride() and value.dtype == key.dtype
+    assert key.dtype in (torch.float16, torch.bfloat16)
+    assert slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous()
+    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.uint8)
+    if not fp8:
+        assert key_cache.dtype == key.dtype
+    assert value_cache.dtype == key_cache.dtype and key_cache.is_contiguous() and value_cache.is_contiguous()
+    w = _KvWrite()
+    w.num_tokens, w.num_kv_heads, w.head_size = key.shape
+    w.block_size = block_size
+    w.kv_block_stride, w.kv_token_stride, w.kv_head_stride = kv_strides
+    w.src_token_stride, w.src_head_stride = key.stride(0), key.stride(1)
+    w.src_dtype = Q_BF16 if key.dtype == torch.bfloat16 else Q_F16
+    w.cache_dtype = KV_E5M2 if fp8 else KV_SAME_AS_Q
+    w.num_pool_blocks = key_cache.shape[0]
+    w.fp8_scale = fp8_scale
+    lib().oracle_kv_cache_write(_ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache),
+                                _ptr(slot_mapping), ctypes.byref(w))
 
 
 def num_threads() -> int:

@@ -21,13 +21,15 @@ def L():
 
 
 def test_header_symbols_are_exported(L):
-    header = open(os.path.join(ROOT, "include", "fa_paged_attention.h")).read()
-    body = header[header.index('extern "C"'):]
-    declared = set(re.findall(r"\b(fa_[a-z0-9_]+)\s*\(", body))
+    declared = set()
+    for name in ("fa_paged_attention.h", "fa_kv_cache.h"):
+        header = open(os.path.join(ROOT, "include", name)).read()
+        body = header[header.index('extern "C"'):]
+        declared |= set(re.findall(r"\b(fa_[a-z0-9_]+)\s*\(", body))
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 1
+    assert L.fa_paged_attention_abi_version() == 2
 
 
 def test_struct_layouts_match_header():
@@ -36,6 +38,8 @@ def test_struct_layouts_match_header():
     assert _cabi.Shape.kv_block_stride.offset == 32
     assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4
     assert _cabi.Options.elapsed_us.offset == 32
+    assert ctypes.sizeof(_cabi.KvWriteShape) == 4 * 4 + 5 * 8 + 2 * 4 + 8
+    assert _cabi.KvWriteShape.src_dtype.offset == 56 and _cabi.KvWriteShape.num_pool_blocks.offset == 64
 
 
 def _shape(**kw):
@@ -120,3 +124,33 @@ def test_workload_generators_are_deterministic():
     g = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=64, seqlen_k=339, varlen=True, has_sinks=True)
     assert g.partition_size == 256 and g.key_cache.shape == (12, 64, 2, 64)
     assert int(g.context_lens.min()) >= 319 and int(g.context_lens.max()) <= 339
+
+
+def _kv_write(L, ptr=0x1000, slots=0x1000, **kw):
+    sh = _cabi.KvWriteShape()
+    base = dict(num_tokens=4, num_kv_heads=2, head_size=128, block_size=16,
+                kv_block_stride=2 * 16 * 128, kv_token_stride=128, kv_head_stride=16 * 128,
+                src_token_stride=0, src_head_stride=0, src_dtype=_cabi.FA_DTYPE_F16,
+                cache_dtype=_cabi.FA_KV_CACHE_E5M2, num_pool_blocks=8)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(sh, k, v)
+    op = _cabi.Options()
+    op.validate_only = 1
+    return L.fa_kv_cache_write(ptr, ptr, ptr, ptr, slots, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
+
+
+def test_kv_cache_write_argument_checks(L):
+    assert _kv_write(L) == (_cabi.FA_OK, "")
+    assert _kv_write(L, cache_dtype=_cabi.FA_KV_CACHE_16BIT, src_dtype=_cabi.FA_DTYPE_BF16)[0] == _cabi.FA_OK
+    assert _kv_write(L, ptr=0)[0] == _cabi.FA_ERR_NULL_POINTER
+    assert _kv_write(L, slots=0)[0] == _cabi.FA_ERR_NULL_POINTER
+    assert _kv_write(L, src_dtype=5)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
+    assert _kv_write(L, cache_dtype=2)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
+    assert _kv_write(L, head_size=100)[0] == _cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE
+    assert _kv_write(L, num_pool_blocks=0)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _kv_write(L, kv_token_stride=64)[0] == _cabi.FA_ERR_BAD_SHAPE       # shorter than a row
+    assert _kv_write(L, kv_head_stride=16 * 128 + 4)[0] == _cabi.FA_ERR_BAD_SHAPE  # misaligned
+    assert _kv_write(L, src_token_stride=100)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _kv_write(L, ptr=0x1008)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _kv_write(L, num_tokens=0)[0] == _cabi.FA_OK
