@@ -14,6 +14,9 @@ roofline     per-kernel HIP-event time on the launch stream (the library's own
 cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTorch
              reference) on the same workload on this box's host cores
 configs      the other four configurations, each timed the same way
+kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
+             rounding): kernel time by the same events, read + written bytes against the
+             HBM peak, and its CPU oracle on a bounded sample
 """
 from __future__ import annotations
 
@@ -110,6 +113,50 @@ def _cpu_baseline(index, torch, W, budget_s=12.0):
                        f"oracle_attention_ref, {dt:.1f} s")
 
 
+def _time_kv_cache_write(steps, torch, dev, cpu_leg):
+    """Prefill-sized batch of the KV-cache writer: 32768 new tokens x 8 kv heads x 128, fp16
+    rows into E5M2 head-major pools of 65536 16-token blocks, random free slots.  Six
+    source/pool sets rotate (1.6 GB between two uses of the same bytes)."""
+    from flash_attention_factory_amd.lib import kv_cache_write
+    N, Hk, D, B, NB, R = 32768, 8, 128, 16, 65536, 6
+    g = torch.Generator(device=dev).manual_seed(0)
+    keys = [torch.randn(N, Hk, D, generator=g, device=dev, dtype=torch.float16) for _ in range(R)]
+    vals = [torch.randn(N, Hk, D, generator=g, device=dev, dtype=torch.float16) for _ in range(R)]
+    pools = [(torch.zeros((NB, Hk, B, D), dtype=torch.uint8, device=dev),
+              torch.zeros((NB, Hk, B, D), dtype=torch.uint8, device=dev)) for _ in range(R)]
+    slots = [torch.randperm(NB * B, generator=g, device=dev)[:N].to(torch.int64) for _ in range(R)]
+    view = lambda t: t.permute(0, 2, 1, 3).view(torch.float8_e5m2)
+    ts = []
+    for it in range(5 + steps):
+        k = it % R
+        t = kv_cache_write.run(keys[k], vals[k], view(pools[k][0]), view(pools[k][1]), slots[k])
+        if it >= 5:
+            ts.append(t[0])
+    us = float(torch.tensor(ts, dtype=torch.float64).mean())
+    read_b, write_b = 2 * N * Hk * D * 2 + 8 * N, 2 * N * Hk * D
+    res = dict(workload=f"kv_cache_write: {N} tokens x {Hk} kv heads x {D}, fp16 -> E5M2, head-major pool of "
+                        f"{NB} blocks of {B}, random slots",
+               kernel="kv_cache_write_kernel<F16, e5m2>", steps=steps, us_per_call=us,
+               read_bytes=read_b, write_bytes=write_b, gbps_kernels=(read_b + write_b) / us / 1e3,
+               hbm_frac=(read_b + write_b) / us / 1e3 / HBM_PEAK_GBPS)
+    if cpu_leg:
+        from oracle import oracle as O
+        n = 2048
+        kc = torch.zeros((n // B, Hk, B, D), dtype=torch.uint8)
+        vc = torch.zeros_like(kc)
+        kh, vh = keys[0][:n].cpu(), vals[0][:n].cpu()
+        sl = torch.randperm(n, dtype=torch.int64)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 3.0:
+            O.kv_cache_write(kh, vh, kc, vc, sl, block_size=B, kv_strides=(Hk * B * D, D, B * D))
+            reps += 1
+        per = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = dict(value=(read_b + write_b) * (n / N) / per / 1e9, unit="GB/s", cores=1, kind="port",
+                                   sample=f"{n} of the {N} tokens, {reps} repetitions of oracle_kv_cache_write")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,6 +165,7 @@ def main():
     ap.add_argument("--configs", type=str, default="0,2,3,4",
                     help="other configurations to time besides configuration 1 ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kv-cache-write", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no multi-GPU form in this build "
@@ -173,6 +221,10 @@ def main():
                      "kernel_us": kernel_us},
         "configs": others,
     }
+    if not args.no_kv_cache_write:
+        del built
+        torch.cuda.empty_cache()
+        line["kv_cache_write"] = _time_kv_cache_write(max(20, args.steps // 2), torch, dev, not args.no_cpu_baseline)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(1, torch, W)
     print(json.dumps(line), flush=True)

@@ -7,8 +7,13 @@
 //
 // One thread moves 8 consecutive head-dim elements of one (token, kv head) row of K and
 // of V: a 16-byte load each, a 16-byte (16-bit pool) or 8-byte (E5M2 pool) store each.
-// The 16 (head 128) or 8 (head 64) threads of a row sit next to each other, so loads and
-// stores of a row are one contiguous segment.
+// The threads of a row sit next to each other, so loads and stores of a row are one
+// contiguous segment.  A work-group covers 256 / (pieces per token) whole tokens, so a
+// thread's place inside the token (kv head, piece of the row) costs two small divisions
+// and the slot one shift.  One work-group per token group, nothing looped or unrolled:
+// measured, a resident grid striding over tokens with 1, 2 or 4 tokens in flight per
+// thread is 3-18 % slower -- a read stream mixed with a write stream wants less in flight,
+// not more.
 #pragma once
 
 #include <type_traits>
@@ -23,55 +28,27 @@ struct KvWriteParams {
   char *key_cache;
   char *value_cache;
   const int64_t *slot_mapping;
-  float inv_scale;          // 1 / fp8_scale
-  int32_t num_kv_heads;
-  int32_t pieces_per_row;   // head_size / 8
-  int64_t total_pieces;     // num_tokens * num_kv_heads * pieces_per_row
+  float inv_scale;            // 1 / fp8_scale
+  int32_t num_tokens;
+  int32_t pieces_per_row;     // head_size / 8
+  int32_t pieces_per_token;   // num_kv_heads * pieces_per_row
+  int32_t tokens_per_group;   // tokens one work-group covers per step: max(1, 256 / pieces_per_token)
   int32_t block_size;
-  int64_t num_slots;        // num_pool_blocks * block_size
-  int64_t kv_block_bytes;   // pool strides in BYTES
+  int32_t block_shift;        // log2(block_size), or -1 if block_size is no power of two
+  uint32_t num_slots;         // num_pool_blocks * block_size
+  int64_t kv_block_bytes;     // pool strides in BYTES
   int64_t kv_token_bytes;
   int64_t kv_head_bytes;
-  int64_t src_token_bytes;  // source strides in BYTES
+  int64_t src_token_bytes;    // source strides in BYTES
   int64_t src_head_bytes;
 };
 
-// Two fp16 values in one dword -> their two E5M2 bytes in bits 0..7 and 16..23.
-// E5M2 is binary16 cut to its top byte, so rounding to nearest even is an integer add on
-// the magnitude bits: + 0x7f + (lowest kept bit).  A carry out of the mantissa moves into
-// the exponent, which is exactly what rounding up to the next binade -- or to infinity --
-// needs, and binary16 subnormals land on E5M2 subnormals the same way.  NaN keeps a
-// non-zero mantissa (0x7f) and its sign.
-__device__ __forceinline__ uint32_t e5m2_from_f16_pair(uint32_t w) {
-  const uint32_t mag = w & 0x7fff7fffu;
-  const uint32_t sign = (w >> 8) & 0x00800080u;
-  const uint32_t odd = (mag >> 8) & 0x00010001u;
-  const uint32_t rounded = ((mag + 0x007f007fu + odd) >> 8) & 0x00ff00ffu;
-  const uint32_t is_nan = ((mag + 0x03ff03ffu) >> 15) & 0x00010001u;  // magnitude above 0x7c00
-  const uint32_t nan_mask = is_nan * 0xffu;
-  return ((rounded & ~nan_mask) | (is_nan * 0x7fu)) | sign;
-}
-
-// One fp32 value -> its E5M2 byte, rounded once (to nearest even).  Used where the value
-// is not an fp16 to begin with (bf16 sources) or has been scaled, so that no second
-// rounding through fp16 can creep in.
-__device__ __forceinline__ uint32_t e5m2_from_f32(float f) {
+// fp32 -> E5M2 byte exactly as the tensor cast does it, in software: round to nearest
+// even, 65536 and beyond (infinity included) to infinity, NaN to 0x7f with its sign.
+// Only NaN ever comes here; everything else goes through the conversion instruction.
+__device__ __forceinline__ uint32_t e5m2_nan_or_keep(float f, uint32_t converted) {
   const uint32_t x = __builtin_bit_cast(uint32_t, f);
-  const uint32_t sign = (x >> 24) & 0x80u;
-  const uint32_t mag = x & 0x7fffffffu;
-  uint32_t r;
-  if (mag < 0x38800000u) {
-    // below 2^-14: E5M2 subnormals are multiples of 2^-16, which is the spacing of fp32
-    // in [128, 256) -- adding 128 makes the fp32 adder do the rounding
-    r = __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, mag) + 128.0f) - 0x43000000u;
-  } else {
-    // keep 2 mantissa bits: add half of the dropped 21 bits (less one, plus the lowest kept
-    // bit, for ties to even), re-bias the exponent from 127 to 15
-    r = (mag + 0x000fffffu + ((mag >> 21) & 1u) - (112u << 23)) >> 21;
-  }
-  r = mag >= 0x47800000u ? 0x7cu : r;  // 65536 and beyond, infinity included
-  r = mag > 0x7f800000u ? 0x7fu : r;   // NaN
-  return r | sign;
+  return (x & 0x7fffffffu) > 0x7f800000u ? (0x7fu | ((x >> 24) & 0x80u)) : converted;
 }
 
 template <typename ST>
@@ -84,50 +61,76 @@ __device__ __forceinline__ float f32_from_half_of(uint32_t w, int hi) {
   }
 }
 
-// 8 source elements (4 dwords) -> 8 E5M2 bytes (2 dwords).
+// 8 source elements (4 dwords) -> 8 E5M2 bytes (2 dwords).  v_cvt_pk_bf8_f32 rounds two
+// fp32 values to nearest even, sends what lies beyond the E5M2 range to infinity and
+// handles subnormals -- checked against the tensor cast on every fp16 and bf16 input --
+// but it has its own NaN pattern, so NaN bytes (exponent 31, mantissa not 0) are spotted
+// in the result and rewritten to the cast's 0x7f | sign.
 template <typename ST, bool SCALED>
 __device__ __forceinline__ u32x2 e5m2_from_row_piece(u32x4 src, float mul) {
-  uint32_t b[4];  // bytes of elements 2k and 2k+1 at bits 0..7 and 16..23
+  float f[8];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    if constexpr (std::is_same<ST, F16>::value && !SCALED) {
-      b[k] = e5m2_from_f16_pair(src[k]);
-    } else {
-      b[k] = e5m2_from_f32(f32_from_half_of<ST>(src[k], 0) * mul) |
-             (e5m2_from_f32(f32_from_half_of<ST>(src[k], 1) * mul) << 16);
-    }
+    f[2 * k] = f32_from_half_of<ST>(src[k], 0);
+    f[2 * k + 1] = f32_from_half_of<ST>(src[k], 1);
   }
-  // gather bytes 0 and 2 of b[0], b[1] into one dword, and of b[2], b[3] into the next
+  if constexpr (SCALED) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) f[k] *= mul;
+  }
   u32x2 out;
-  out[0] = __builtin_amdgcn_perm(b[1], b[0], 0x06040200u);
-  out[1] = __builtin_amdgcn_perm(b[3], b[2], 0x06040200u);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h], f[4 * h + 1], 0, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h + 2], f[4 * h + 3], w, true);
+    uint32_t u = (uint32_t)w;
+    // any byte with magnitude bits above 0x7c is a NaN
+    if ((((u & 0x7f7f7f7fu) + 0x03030303u) & 0x80808080u) != 0) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t b = e5m2_nan_or_keep(f[4 * h + e], (u >> (8 * e)) & 0xffu);
+        u = (u & ~(0xffu << (8 * e))) | (b << (8 * e));
+      }
+    }
+    out[h] = u;
+  }
   return out;
 }
 
 template <typename ST, bool KV8, bool SCALED>
 __global__ void __launch_bounds__(256) kv_cache_write_kernel(const KvWriteParams p) {
-  const int64_t piece = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (piece >= p.total_pieces) return;
-  const int64_t row = piece / p.pieces_per_row;
-  const int part = (int)(piece - row * p.pieces_per_row);
-  const int64_t token = row / p.num_kv_heads;
-  const int head = (int)(row - token * p.num_kv_heads);
-  const int64_t slot = p.slot_mapping[token];
-  if (slot < 0 || slot >= p.num_slots) return;  // padding token
-  const int64_t block = slot / p.block_size;
-  const int64_t offset = slot - block * p.block_size;
+  const int ppt = p.pieces_per_token;
+  // place inside the group of tokens a work-group covers per step
+  const int local_token = (int)threadIdx.x / ppt;  // 0 when a token has more pieces than threads
+  if (local_token >= p.tokens_per_group) return;
+  const int q_first = (int)threadIdx.x - local_token * ppt;
+  const int64_t token_stride = (int64_t)gridDim.x * p.tokens_per_group;
 
-  const int64_t src = token * p.src_token_bytes + head * p.src_head_bytes + part * 16;
-  const u32x4 k = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.key + src));
-  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.value + src));
-  const int64_t dst = block * p.kv_block_bytes + offset * p.kv_token_bytes + head * p.kv_head_bytes +
-                      part * (KV8 ? 8 : 16);
-  if constexpr (KV8) {
-    *reinterpret_cast<u32x2 *>(p.key_cache + dst) = e5m2_from_row_piece<ST, SCALED>(k, p.inv_scale);
-    *reinterpret_cast<u32x2 *>(p.value_cache + dst) = e5m2_from_row_piece<ST, SCALED>(v, p.inv_scale);
-  } else {
-    *reinterpret_cast<u32x4 *>(p.key_cache + dst) = k;
-    *reinterpret_cast<u32x4 *>(p.value_cache + dst) = v;
+  for (int q = q_first; q < ppt; q += 256) {  // one trip unless a token has more than 256 pieces
+    const int head = q / p.pieces_per_row;
+    const int part = q - head * p.pieces_per_row;
+    const int64_t src_off = (int64_t)head * p.src_head_bytes + part * 16;
+    const int64_t dst_off = (int64_t)head * p.kv_head_bytes + part * (KV8 ? 8 : 16);
+    // one trip as well unless the batch needs more work-groups than a grid holds
+    for (int64_t token = (int64_t)blockIdx.x * p.tokens_per_group + local_token; token < p.num_tokens;
+         token += token_stride) {
+      const int64_t slot = p.slot_mapping[token];
+      const int64_t src = token * p.src_token_bytes + src_off;
+      const u32x4 k = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.key + src));
+      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.value + src));
+      if (slot < 0 || slot >= (int64_t)p.num_slots) continue;  // padding token
+      const uint32_t s = (uint32_t)slot;
+      const uint32_t block = p.block_shift >= 0 ? s >> p.block_shift : s / (uint32_t)p.block_size;
+      const uint32_t row = s - block * (uint32_t)p.block_size;
+      const int64_t dst = (int64_t)block * p.kv_block_bytes + (int64_t)row * p.kv_token_bytes + dst_off;
+      if constexpr (KV8) {
+        *reinterpret_cast<u32x2 *>(p.key_cache + dst) = e5m2_from_row_piece<ST, SCALED>(k, p.inv_scale);
+        *reinterpret_cast<u32x2 *>(p.value_cache + dst) = e5m2_from_row_piece<ST, SCALED>(v, p.inv_scale);
+      } else {
+        *reinterpret_cast<u32x4 *>(p.key_cache + dst) = k;
+        *reinterpret_cast<u32x4 *>(p.value_cache + dst) = v;
+      }
+    }
   }
 }
 

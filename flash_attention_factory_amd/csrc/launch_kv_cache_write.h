@@ -6,6 +6,8 @@
 
 #include "../../include/fa_kv_cache.h"
 #include "kv_cache_write_kernel.h"
+#include <algorithm>
+
 #include "launch_common.h"
 
 namespace fa {
@@ -48,6 +50,12 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
     return FA_OK;
   }
 
+  const int64_t num_slots = s->num_pool_blocks * s->block_size;
+  if (num_slots > 0xffffffffLL)
+    return fail(FA_ERR_BAD_SHAPE, "pools of more than 2^32 - 1 token slots are not supported");
+  const int64_t pieces_per_token = (int64_t)s->num_kv_heads * (s->head_size / 8);
+  if (pieces_per_token > 0x7fffffff) return fail(FA_ERR_BAD_SHAPE, "num_kv_heads * head_size is too large");
+
   KvWriteParams p;
   p.key = reinterpret_cast<const char *>(key);
   p.value = reinterpret_cast<const char *>(value);
@@ -56,33 +64,34 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   p.slot_mapping = slot_mapping;
   const float scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
   p.inv_scale = 1.0f / scale;
-  p.num_kv_heads = s->num_kv_heads;
+  p.num_tokens = s->num_tokens;
   p.pieces_per_row = s->head_size / 8;
-  p.total_pieces = (int64_t)s->num_tokens * s->num_kv_heads * p.pieces_per_row;
+  p.pieces_per_token = (int32_t)pieces_per_token;
+  p.tokens_per_group = (int32_t)std::max<int64_t>(1, 256 / pieces_per_token);
   p.block_size = s->block_size;
-  p.num_slots = s->num_pool_blocks * s->block_size;
+  p.block_shift = is_pow2(s->block_size) ? ilog2(s->block_size) : -1;
+  p.num_slots = (uint32_t)num_slots;
   p.kv_block_bytes = s->kv_block_stride * eb;
   p.kv_token_bytes = s->kv_token_stride * eb;
   p.kv_head_bytes = s->kv_head_stride * eb;
   p.src_token_bytes = src_token * 2;
   p.src_head_bytes = src_head * 2;
-  const int64_t groups = (p.total_pieces + 255) / 256;
-  if (groups > 0x7fffffff) return fail(FA_ERR_BAD_SHAPE, "too many elements for one launch");
 
   hipStream_t stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   KernelTimer timer(o && o->elapsed_us, stream);
-  const dim3 grid((unsigned)groups), block(256);
+  // one work-group per group of tokens (the kernel strides if a grid cannot hold them all)
+  const int64_t groups_needed = ((int64_t)s->num_tokens + p.tokens_per_group - 1) / p.tokens_per_group;
+  const dim3 grid((unsigned)std::min<int64_t>(groups_needed, 0x7fffffff)), block(256);
   const bool bf16 = s->src_dtype == FA_DTYPE_BF16;
   const bool scaled = scale != 1.0f;
-  if (!kv8) {
+  if (!kv8) {  // a 16-bit pool takes bit copies whatever the 16-bit type
     FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, false, false>, grid, block, 0, p));
   } else if (bf16) {
-    // the bf16 path multiplies in fp32 anyway
-    FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<BF16, true, true>, grid, block, 0, p));
-  } else if (scaled) {
-    FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, true>, grid, block, 0, p));
+    if (scaled) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<BF16, true, true>, grid, block, 0, p));
+    else FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<BF16, true, false>, grid, block, 0, p));
   } else {
-    FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, false>, grid, block, 0, p));
+    if (scaled) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, true>, grid, block, 0, p));
+    else FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, false>, grid, block, 0, p));
   }
   if (o && o->elapsed_us) FA_HIP_CHECK(timer.read(0, &o->elapsed_us[0]));
   return FA_OK;
