@@ -14,6 +14,8 @@ roofline     per-kernel HIP-event time on the launch stream (the library's own
 cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTorch
              reference) on the same workload on this box's host cores
 configs      the other four configurations, each timed the same way
+stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
+             the asynchronous torch.library operators, and a HIP-graph replay of them
 kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
              rounding): kernel time by the same events, read + written bytes against the
              HBM peak, and its CPU oracle on a bounded sample
@@ -157,6 +159,59 @@ def _time_kv_cache_write(steps, torch, dev, cpu_leg):
     return res
 
 
+def _time_stream_ordered(steps, torch, W, runner, dev):
+    """Host cost of one small decode step (configuration 0: KV-cache append of one token per
+    sequence, then the loop kernel) three ways: the timed `run` calls, which block on every
+    kernel as upstream's launchers do; the torch.library operators, asynchronous on the
+    current stream; and the same two operators replayed from a HIP graph."""
+    from flash_attention_factory_amd import torch_ops  # noqa: F401
+    from flash_attention_factory_amd.lib import kv_cache_write, paged_attention_loop
+    ops = torch.ops.fa_amd
+    w = W.make_config(0, device=dev, pools_on_device=True)
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    kv, vv = (w.key_cache.permute(0, 2, 1, 3), w.value_cache.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR \
+        else (w.key_cache, w.value_cache)
+    bufs = runner.alloc_buffers(w)
+    key = torch.randn((S, Hk, D), device=dev).to(w.query.dtype)
+    value = torch.randn((S, Hk, D), device=dev).to(w.query.dtype)
+    last = (w.context_lens - 1).long()
+    slots = w.block_tables.gather(1, (last // B)[:, None]).squeeze(1).long() * B + last % B
+
+    def blocking():
+        kv_cache_write.run(key, value, kv, vv, slots)
+        paged_attention_loop.run(None, None, None, bufs.out, None, w.query, kv, vv, w.block_tables, w.context_lens,
+                                 H // Hk, w.scale, B, 0, None, w.sinks, 0.0)
+
+    def asynchronous():
+        ops.kv_cache_write(key, value, kv, vv, slots, 1.0)
+        ops.paged_attention_loop(bufs.out, w.query, kv, vv, w.block_tables, w.context_lens, w.scale, w.sinks)
+
+    def wall(fn, n):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    res = dict(workload="config0 decode step: kv_cache_write of 1 token per sequence + loop kernel (S4 H8 D64)",
+               us_per_step_blocking=wall(blocking, steps), us_per_step_async_ops=wall(asynchronous, steps))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        asynchronous()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        asynchronous()
+    res["us_per_step_graph_replay"] = wall(graph.replay, steps)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -221,6 +276,7 @@ def main():
                      "kernel_us": kernel_us},
         "configs": others,
     }
+    line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
         del built
         torch.cuda.empty_cache()

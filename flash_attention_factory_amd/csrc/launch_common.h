@@ -201,14 +201,14 @@ class KernelTimer {
   // Launch `kernel` on the stream; with timing on, events 2*slot / 2*slot+1 bracket it.
   template <typename Params>
   hipError_t launch(void (*kernel)(Params), dim3 grid, dim3 block, int slot, const Params &prm) {
-    hipEvent_t start = nullptr, stop = nullptr;
-    if (enabled_) {
-      hipError_t e = ensure();
-      if (e != hipSuccess) return e;
-      start = events()[2 * slot];
-      stop = events()[2 * slot + 1];
+    if (!enabled_) {  // plain launch: nothing but the kernel goes on the stream, so a
+                      // caller may record it into a HIP graph
+      hipLaunchKernelGGL(kernel, grid, block, 0, stream_, prm);
+      return hipGetLastError();
     }
-    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream_, start, stop, 0, prm);
+    hipError_t e = ensure();
+    if (e != hipSuccess) return e;
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream_, events()[2 * slot], events()[2 * slot + 1], 0, prm);
     return hipGetLastError();
   }
 

@@ -1,0 +1,94 @@
+"""Stream-ordered ``torch.library`` operators over the C ABI.
+
+Upstream's launchers build a queue of their own and block on every kernel
+(launch_kernels_reduce.h:35-38 creates ``sycl::queue q``; the line that would have taken
+PyTorch's current stream, ``c10::xpu::getCurrentXPUStream().queue()``, is commented out at
+:35; ``event1.wait()`` :56 and ``event2.wait()`` :75 stall the host between kernels).  The
+operators below are what that commented-out line was after: each one enqueues its kernels on
+PyTorch's *current* stream and returns at once -- no event, no synchronisation, nothing but
+kernel launches on the stream -- so they order with the rest of a model's work and can be
+recorded into a HIP graph (``torch.cuda.graph``) and replayed.
+
+    torch.ops.fa_amd.paged_attention_loop(out, query, key_cache, value_cache, block_tables,
+                                          context_lens, scale, sinks)
+    torch.ops.fa_amd.paged_attention_reduce(out, exp_sums, max_logits, tmp_out, query, key_cache,
+                                            value_cache, block_tables, context_lens, scale,
+                                            partition_size, sinks)
+    torch.ops.fa_amd.paged_attention_fp8_loop(..., scale, fp8_scale, sinks)
+    torch.ops.fa_amd.paged_attention_fp8_reduce(..., scale, fp8_scale, partition_size, sinks)
+    torch.ops.fa_amd.kv_cache_write(key, value, key_cache, value_cache, slot_mapping, fp8_scale)
+
+Caches are ``[blocks, block_size, kv_heads, head_size]`` views as in ``lib.*.run``; every
+output is an argument the operator mutates, nothing is allocated.  Importing this module
+registers the operators; there is no CPU implementation.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from .lib import (kv_cache_write as _kv_cache_write, paged_attention_fp8_loop as _fp8_loop,
+                  paged_attention_fp8_reduce as _fp8_reduce, paged_attention_loop as _loop,
+                  paged_attention_reduce as _reduce)
+
+_NS = "fa_amd"
+
+
+def _group(query: Tensor, key_cache: Tensor) -> int:
+    return query.size(1) // key_cache.size(2)
+
+
+@torch.library.custom_op(f"{_NS}::paged_attention_loop", mutates_args=("out",), device_types="cuda")
+def paged_attention_loop(out: Tensor, query: Tensor, key_cache: Tensor, value_cache: Tensor,
+                         block_tables: Tensor, context_lens: Tensor, scale: float,
+                         sinks: Optional[Tensor] = None) -> None:
+    _loop.run(None, None, None, out, None, query, key_cache, value_cache, block_tables, context_lens,
+              _group(query, key_cache), scale, key_cache.size(1), 0, None, sinks, 0.0, timed=False)
+
+
+@torch.library.custom_op(f"{_NS}::paged_attention_fp8_loop", mutates_args=("out",), device_types="cuda")
+def paged_attention_fp8_loop(out: Tensor, query: Tensor, key_cache: Tensor, value_cache: Tensor,
+                             block_tables: Tensor, context_lens: Tensor, scale: float, fp8_scale: float,
+                             sinks: Optional[Tensor] = None) -> None:
+    _fp8_loop.run(None, None, None, out, None, query, key_cache, value_cache, block_tables, context_lens,
+                  _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, None, sinks, 0.0,
+                  timed=False)
+
+
+@torch.library.custom_op(f"{_NS}::paged_attention_reduce",
+                         mutates_args=("out", "exp_sums", "max_logits", "tmp_out"), device_types="cuda")
+def paged_attention_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tmp_out: Tensor, query: Tensor,
+                           key_cache: Tensor, value_cache: Tensor, block_tables: Tensor, context_lens: Tensor,
+                           scale: float, partition_size: int = 0, sinks: Optional[Tensor] = None) -> None:
+    if tmp_out.dtype != torch.float32:
+        raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
+    _reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
+                context_lens, _group(query, key_cache), scale, key_cache.size(1), 0, None, sinks, 0.0,
+                partition_size=partition_size, timed=False)
+
+
+@torch.library.custom_op(f"{_NS}::paged_attention_fp8_reduce",
+                         mutates_args=("out", "exp_sums", "max_logits", "tmp_out"), device_types="cuda")
+def paged_attention_fp8_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tmp_out: Tensor, query: Tensor,
+                               key_cache: Tensor, value_cache: Tensor, block_tables: Tensor,
+                               context_lens: Tensor, scale: float, fp8_scale: float, partition_size: int = 0,
+                               sinks: Optional[Tensor] = None) -> None:
+    if tmp_out.dtype != torch.float32:
+        raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
+    _fp8_reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
+                    context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, None, sinks,
+                    0.0, partition_size=partition_size, timed=False)
+
+
+@torch.library.custom_op(f"{_NS}::kv_cache_write", mutates_args=("key_cache", "value_cache"), device_types="cuda")
+def kv_cache_write(key: Tensor, value: Tensor, key_cache: Tensor, value_cache: Tensor, slot_mapping: Tensor,
+                   fp8_scale: float = 1.0) -> None:
+    _kv_cache_write.run(key, value, key_cache, value_cache, slot_mapping, fp8_scale, timed=False)
+
+
+# Shape propagation for tracing: every operator only writes into its arguments.
+for _op in (paged_attention_loop, paged_attention_fp8_loop, paged_attention_reduce, paged_attention_fp8_reduce,
+            kv_cache_write):
+    _op.register_fake(lambda *args, **kwargs: None)

@@ -1,0 +1,115 @@
+"""The stream-ordered torch.library operators: same results as the timed ``lib.*.run`` calls,
+and a HIP graph holding a whole decode step (KV-cache append, FP8 loop decode, FP8 split
+decode) replays correctly.  The graph is replayed several times with the program's own eager
+work and synchronisations between the replays, and every replay is checked against eager."""
+import pytest
+import torch
+
+from flash_attention_factory_amd import runner, workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")
+
+
+def _views(w, kc, vc):
+    """[blocks, block_size, kv_heads, head_size] views of pools stored in the workload's layout."""
+    if w.layout == W.HEAD_MAJOR:
+        return kc.permute(0, 2, 1, 3), vc.permute(0, 2, 1, 3)
+    return kc, vc
+
+
+@pytest.mark.parametrize("index", [0, 3])
+def test_operators_match_the_run_functions(index):
+    from flash_attention_factory_amd import torch_ops  # noqa: F401  (registers the operators)
+    dev = _dev()
+    w = W.make_config(index, num_seqs=4, pool_blocks=300, lens=[100, 700, 33, 512]).to(dev)
+    fp8 = w.is_fp8
+    kv, vv = _views(w, w.key_cache, w.value_cache)
+    ref_loop = runner.alloc_buffers(w)
+    runner.run_workload(w, "fp8_loop" if fp8 else "loop", ref_loop)
+    ref_split = runner.alloc_buffers(w)
+    runner.run_workload(w, "fp8_reduce" if fp8 else "reduce", ref_split)
+    got = runner.alloc_buffers(w)
+    ops = torch.ops.fa_amd
+    if fp8:
+        ops.paged_attention_fp8_loop(got.out, w.query, kv, vv, w.block_tables, w.context_lens, w.scale, w.fp8_scale, w.sinks)
+    else:
+        ops.paged_attention_loop(got.out, w.query, kv, vv, w.block_tables, w.context_lens, w.scale, w.sinks)
+    torch.cuda.synchronize()
+    assert torch.equal(got.out, ref_loop.out)
+    got.out.zero_()
+    if fp8:
+        ops.paged_attention_fp8_reduce(got.out, got.exp_sums, got.max_logits, got.tmp_out, w.query, kv, vv,
+                                       w.block_tables, w.context_lens, w.scale, w.fp8_scale, w.partition_size, w.sinks)
+    else:
+        ops.paged_attention_reduce(got.out, got.exp_sums, got.max_logits, got.tmp_out, w.query, kv, vv,
+                                   w.block_tables, w.context_lens, w.scale, w.partition_size, w.sinks)
+    torch.cuda.synchronize()
+    assert torch.equal(got.out, ref_split.out)
+
+
+def test_decode_step_in_a_hip_graph():
+    from flash_attention_factory_amd import torch_ops  # noqa: F401
+    dev = _dev()
+    ops = torch.ops.fa_amd
+    w = W.make_config(3, num_seqs=4, pool_blocks=300, lens=[100, 700, 33, 512]).to(dev)   # E5M2 pools, fp16 queries
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    gen = torch.Generator(device=dev).manual_seed(1)
+
+    def fresh_state():
+        kc, vc = w.key_cache.clone(), w.value_cache.clone()
+        bufs_a, bufs_b = runner.alloc_buffers(w), runner.alloc_buffers(w)
+        return dict(kc=kc, vc=vc, views=_views(w, kc, vc), ctx=w.context_lens.clone(), query=w.query.clone(),
+                    key=torch.zeros((S, Hk, D), dtype=torch.float16, device=dev),
+                    value=torch.zeros((S, Hk, D), dtype=torch.float16, device=dev),
+                    slots=torch.zeros(S, dtype=torch.int64, device=dev), loop=bufs_a, split=bufs_b)
+
+    def step(st):  # append one token per sequence, then decode it twice (loop and split kernels)
+        ops.kv_cache_write(st["key"], st["value"], st["views"][0], st["views"][1], st["slots"], 1.0)
+        ops.paged_attention_fp8_loop(st["loop"].out, st["query"], st["views"][0], st["views"][1], w.block_tables,
+                                     st["ctx"], w.scale, 1.0, None)
+        ops.paged_attention_fp8_reduce(st["split"].out, st["split"].exp_sums, st["split"].max_logits,
+                                       st["split"].tmp_out, st["query"], st["views"][0], st["views"][1],
+                                       w.block_tables, st["ctx"], w.scale, 1.0, w.partition_size, None)
+
+    def new_inputs(st):  # in place, so that a graph holding these tensors sees them
+        old = st["ctx"].clone()
+        st["slots"].copy_(w.block_tables.gather(1, (old // B).long()[:, None]).squeeze(1).long() * B + old % B)
+        st["ctx"].add_(1)
+        st["key"].copy_(torch.randn((S, Hk, D), generator=gen, device=dev).half())
+        st["value"].copy_(torch.randn((S, Hk, D), generator=gen, device=dev).half())
+        st["query"].copy_(torch.randn((S, H, D), generator=gen, device=dev).half())
+
+    eager, graphed = fresh_state(), fresh_state()
+    # warm-up outside the capture (first calls query occupancy and create nothing afterwards)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        warm = fresh_state()
+        step(warm)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(graphed)
+    for replay in range(4):
+        gen.manual_seed(100 + replay)
+        new_inputs(eager)
+        gen.manual_seed(100 + replay)
+        new_inputs(graphed)
+        step(eager)
+        scratch = torch.randn(1 << 20, device=dev).sum()   # the program's own eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(scratch)
+        assert torch.equal(graphed["loop"].out, eager["loop"].out), f"loop kernel, replay {replay}"
+        assert torch.equal(graphed["split"].out, eager["split"].out), f"split kernels, replay {replay}"
+        assert torch.equal(graphed["kc"].view(torch.uint8), eager["kc"].view(torch.uint8)), f"key pool, replay {replay}"
+        a, b = eager["loop"].out.float(), eager["split"].out.float()
+        assert (a - b).abs().max().item() <= 2.0 ** -9 * a.abs().max().item() + 1e-5
