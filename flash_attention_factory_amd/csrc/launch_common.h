@@ -19,6 +19,7 @@
 #include "paged_attention_persistent_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
+#include "paged_attention_segment_kernel.h"
 
 namespace fa {
 

@@ -30,7 +30,20 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // work-groups as the GPU keeps resident walk the list of live partitions.  Otherwise
   // one work-group per (kv head, partition slot, sequence); slots past a sequence's
   // length return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
-  if (kUsePersistentSplit && shape.num_seqs <= kPersistentMaxSeqs && shape.num_pool_blocks > 0) {
+  int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
+  if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
+      (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
+    // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
+    constexpr int SW = SegmentSplit<KV8>::waves;
+    auto kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KV8, SW, SegmentSplit<KV8>::occ,
+                                            Pipeline<KV8>::tiles_per_chunk>;
+    int resident = 0;
+    FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
+    const int64_t max_items =
+        (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
+    segment_groups = (int)std::min<int64_t>(resident, max_items);
+    FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
+  } else if (kUsePersistentSplit && shape.num_seqs <= kPersistentMaxSeqs && shape.num_pool_blocks > 0) {
     auto kernel = paged_attn_split_persistent_kernel<HEAD_SIZE, QT, KV8, Pipeline<KV8>::occ,
                                                      Pipeline<KV8>::tiles_per_chunk, SplitOrder<KV8>::value>;
     int resident = 0;
@@ -58,11 +71,17 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   rp.max_num_partitions = shape.max_num_partitions;
   rp.partition_size = r.partition_size;
   rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
+  rp.num_seqs = shape.num_seqs;
+  rp.num_kv_heads = shape.num_kv_heads;
+  rp.segment_groups = segment_groups;
   const dim3 rgrid(shape.num_heads, shape.num_seqs);
-  if ((int64_t)shape.num_heads * shape.num_seqs >= kReduceSingleWaveMinPairs) {
-    FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1>, rgrid, dim3(64), 1, rp));
+  const bool one_wave = (int64_t)shape.num_heads * shape.num_seqs >= kReduceSingleWaveMinPairs;
+  if (segment_groups > 0) {
+    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, true>, rgrid, dim3(64), 1, rp));
+    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, true>, rgrid, dim3(256), 1, rp));
   } else {
-    FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4>, rgrid, dim3(256), 1, rp));
+    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, false>, rgrid, dim3(64), 1, rp));
+    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, false>, rgrid, dim3(256), 1, rp));
   }
   if (r.elapsed_us) {
     FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));

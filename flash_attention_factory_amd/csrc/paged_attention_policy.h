@@ -89,6 +89,33 @@ struct SplitOrder {
   static constexpr int value = kKV8 ? FA_SPLIT_ORDER_FP8 : FA_SPLIT_ORDER;
 };
 
+// Split path, segment form: multi-wavefront work-groups take segments of several partitions
+// and write one partial per segment (paged_attention_segment_kernel.h).
+#ifndef FA_SPLIT_SEGMENT
+#define FA_SPLIT_SEGMENT 1
+#endif
+#ifndef FA_SPLIT_SEGMENT_FP8
+#define FA_SPLIT_SEGMENT_FP8 FA_SPLIT_SEGMENT
+#endif
+#ifndef FA_SEGMENT_WAVES
+#define FA_SEGMENT_WAVES 4
+#endif
+#ifndef FA_SEGMENT_OCC
+#define FA_SEGMENT_OCC 2
+#endif
+#ifndef FA_SEGMENT_STREAM_LOADS
+#define FA_SEGMENT_STREAM_LOADS 1
+#endif
+template <bool kKV8>
+struct SegmentSplit {
+  static constexpr bool use = (kKV8 ? FA_SPLIT_SEGMENT_FP8 : FA_SPLIT_SEGMENT) != 0;
+  static constexpr int waves = FA_SEGMENT_WAVES;
+  static constexpr int occ = FA_SEGMENT_OCC;
+  // non-temporal K/V loads: +5 % here for both cache types (long streaming runs per
+  // wavefront, as in the loop kernels)
+  static constexpr bool stream_loads = FA_SEGMENT_STREAM_LOADS != 0;
+};
+
 // Loop path: resident work-groups walk the (sequence, kv head) items, longest first.
 #ifndef FA_PERSISTENT_LOOP
 #define FA_PERSISTENT_LOOP 1

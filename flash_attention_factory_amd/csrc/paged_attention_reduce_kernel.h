@@ -14,6 +14,7 @@
 // wavefronts the partial sums meet in LDS.  Lane j owns D/64 consecutive output elements.
 #pragma once
 
+#include "paged_attention_segment_policy.h"
 #include "paged_attention_utils.h"
 
 namespace fa {
@@ -28,6 +29,11 @@ struct ReduceParams {
   int32_t max_num_partitions;
   int32_t partition_size;
   int32_t max_context;  // max_blocks_per_seq * block_size: lengths are cut to it
+  int32_t num_seqs;
+  int32_t num_kv_heads;
+  int32_t segment_groups;  // work-groups of the segment attention kernel that wrote the partials
+                           // (it wrote one partial per segment of m partitions, into the
+                           // segment's first slot); 0: one partial per partition
 };
 
 constexpr int kReduceRowsInFlight = 16;  // per wavefront and batch
@@ -36,7 +42,7 @@ constexpr int kReduceRowsInFlight = 16;  // per wavefront and batch
 // pairs -- the launch is then short of parallelism and each pair's rows should be in
 // flight at once -- 1 when there are thousands and every wavefront slot of the GPU is
 // filled anyway (no LDS, no barrier, more groups resident).
-template <int D, typename QT, int kReduceWaves>
+template <int D, typename QT, int kReduceWaves, bool SEGMENTS = false>
 __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
   constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
   constexpr int R = kReduceRowsInFlight;
@@ -48,6 +54,16 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;
   np = min(np, p.max_num_partitions);
+  // Partials lie `stride` slots apart: 1, or the segment length the attention kernel chose.
+  int stride = 1;
+  if constexpr (SEGMENTS) {
+    constexpr int NQ = kSegmentMaxSeqs / 64;
+    int ctxv[NQ], parts[NQ];
+    const int total = count_partitions<NQ>(p.context_lens, p.num_seqs, p.max_context, p.partition_size,
+                                           p.max_num_partitions, lane, ctxv, parts);
+    stride = partitions_per_segment(total, p.num_kv_heads, p.segment_groups);
+    np = (np + stride - 1) / stride;  // from here on: the number of partials
+  }
   const int64_t base = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions;
   const float *ml = p.max_logits + base;
   const float *es = p.exp_sums + base;
@@ -64,15 +80,15 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
     for (int u = 0; u < R; ++u) {
       const int q = q0 + wave + kReduceWaves * u;
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * D + e] : 0.f;
+      for (int e = 0; e < EPL; ++e) v[u][e] = (q < np) ? tmp[(int64_t)q * stride * D + e] : 0.f;
     }
   };
   request_rows(0);
   // lane q keeps the scalars of partition q (first group) in registers
-  const float ml0 = (lane < np) ? ml[lane] : -INFINITY;
-  const float es0 = (lane < np) ? es[lane] : 0.f;
+  const float ml0 = (lane < np) ? ml[lane * stride] : -INFINITY;
+  const float es0 = (lane < np) ? es[lane * stride] : 0.f;
   float M = ml0;
-  for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q]);
+  for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q * stride]);
   M = wave_max(M);
 
   float acc[EPL];
@@ -82,7 +98,7 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   for (int g0 = 0; g0 < np; g0 += 64) {
     const int ql = g0 + lane;
     const float w_lane = g0 == 0 ? es0 * __expf(ml0 - M)
-                                 : ((ql < np) ? es[ql] * __expf(ml[ql] - M) : 0.f);
+                                 : ((ql < np) ? es[ql * stride] * __expf(ml[ql * stride] - M) : 0.f);
     W += w_lane;
     for (int b0 = 0; b0 < 64 && g0 + b0 < np; b0 += BATCH) {
       if (g0 + b0 > 0) request_rows(g0 + b0);

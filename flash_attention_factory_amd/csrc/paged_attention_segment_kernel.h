@@ -1,0 +1,296 @@
+// Split-context attention kernel, persistent form with multi-wavefront work-groups.
+//
+// Same role as the other split kernels (upstream paged_attention_kernel_v2.hpp:572-587):
+// partial softmax states go to exp_sums / max_logits / tmp_out and the reduce kernel merges
+// them.  What differs is how much of a sequence one partial covers.  With one partial per
+// 512-token partition a large ragged batch writes thousands of 512-byte rows scattered over
+// the scratch arrays, and a few percent of scattered writes mixed into a saturated read
+// stream cost far more than their bytes.  Here a work-group of NW wavefronts takes a SEGMENT
+// of m consecutive partitions of one (sequence, kv head): its wavefronts interleave the
+// segment's chunks, merge their states in LDS (no barrier: the deferred merge of the
+// persistent loop kernel) and write ONE partial into the slot of the segment's first
+// partition.  The other m - 1 slots are neither written nor read: the reduce kernel is told
+// m and visits slots 0, m, 2m, ...
+//
+// m is chosen on the device from the batch itself -- all wavefronts, and the reduce kernel
+// after them, evaluate partitions_per_segment() on the same context lengths -- so that there
+// are about two segments per resident work-group: a batch of few long sequences is cut
+// finely, in a batch with a thousand (sequence, kv head) pairs most sequences stay whole.
+// Segments are dealt to the work-groups longest first in snake order (see below).
+// Built for up to 256 sequences; larger batches use the grid form.
+#pragma once
+
+#include "paged_attention_kernel.h"
+#include "paged_attention_loop_persistent_kernel.h"
+#include "paged_attention_segment_policy.h"
+
+namespace fa {
+
+template <int D, typename QT, bool KV8, int NW, int OCC, int TPC>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+paged_attn_segment_kernel(const PagedAttnParams p) {
+  using W = WaveAttn<D, QT, KV8, TPC, SegmentSplit<KV8>::stream_loads>;
+  using Chunk = typename W::Chunk;
+  using Ids = typename W::Ids;
+  constexpr int CT = W::CT;
+  constexpr int NR = W::NR;
+  constexpr int NDT = W::NDT;
+  constexpr int SL = NR / NW;
+  constexpr int NQ = kSegmentMaxSeqs / 64;
+  static_assert(NW > 1 && NR % NW == 0 && SL >= 4 && SL % 4 == 0, "each wavefront stores whole 16-byte pieces");
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int S = p.num_seqs;
+  const int Hk = p.num_kv_heads;
+  const int G = gridDim.x;
+  const int max_ctx = p.max_blocks_per_seq << p.block_shift;
+  const int col_max = p.max_blocks_per_seq - 1;
+
+  // ---- segment list, in registers: lane holds sequences lane, lane+64, ... ---------------
+  // Segments are dealt longest first: all full segments (equal length), then the sequences'
+  // last, shorter segments in order of length; work-group j takes positions j, 2G-1-j,
+  // 2G+j, ... of that list (snake order), so the work-groups' totals come out even although
+  // a work-group only gets a handful of segments.
+  int ctxv[NQ], parts[NQ], incl[NQ], fullc[NQ], key[NQ], rank[NQ];
+  const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size,
+                                               p.max_num_partitions, lane, ctxv, parts);
+  const int m = partitions_per_segment(total_parts, Hk, G);
+  const int seg_tokens = m * p.partition_size;
+  int running = 0, tails = 0;
+#pragma unroll
+  for (int j = 0; j < NQ; ++j) {
+    const int cut = min(ctxv[j], parts[j] * p.partition_size);  // what the scratch arrays can hold
+    ctxv[j] = cut;
+    fullc[j] = cut / seg_tokens;
+    const int rem = cut - fullc[j] * seg_tokens;
+    // sort key of the last segment: length, then lower sequence number first; -1: none
+    key[j] = rem > 0 ? (rem << 8) | (255 - (lane + 64 * j)) : -1;
+    rank[j] = 0;
+    int x = fullc[j];
+    if (j * 64 < S) {
+      tails += __builtin_popcountll(__ballot(rem > 0));
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int y = __shfl_up(x, o);
+        if (lane >= o) x += y;
+      }
+    }
+    incl[j] = x + running;
+    running = __builtin_amdgcn_readlane(incl[j], 63);
+  }
+  const int full_total = running;
+  const int total_items = (full_total + tails) * Hk;
+  // rank of every last segment among the last segments (how many are longer)
+#pragma unroll
+  for (int js = 0; js < NQ; ++js) {
+    if (js * 64 < S) {
+      for (int u0 = 0; u0 < min(S - js * 64, 64); u0 += 8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int ku = __builtin_amdgcn_readlane(key[js], u0 + e);
+#pragma unroll
+          for (int jd = 0; jd < NQ; ++jd) rank[jd] += ku > key[jd];
+        }
+      }
+    }
+  }
+
+  struct Item { int seq, kvh, part0, tok_end, c_begin, c_end; };
+  // position in the sorted list -> (sequence, segment, kv head), kv head fastest
+  auto decode = [&](int pos) -> Item {
+    Item it;
+    const int q = __builtin_amdgcn_readfirstlane(pos / Hk);
+    it.kvh = pos - q * Hk;
+    int s = 0;
+    const bool full = q < full_total;
+    if (full) {
+#pragma unroll
+      for (int j = 0; j < NQ; ++j)
+        if (j * 64 < S) s += __builtin_popcountll(__ballot(lane + 64 * j < S && incl[j] <= q));
+    } else {
+      const int rho = q - full_total;
+#pragma unroll
+      for (int j = 0; j < NQ; ++j)
+        if (j * 64 < S) {
+          const unsigned long long hit = __ballot(key[j] >= 0 && rank[j] == rho);
+          if (hit) s = 64 * j + __builtin_ctzll(hit);
+        }
+    }
+    s = min(s, S - 1);
+    int inc_s = 0, full_s = 0, ctx_s = 0;
+#pragma unroll
+    for (int j = 0; j < NQ; ++j)
+      if ((s >> 6) == j) {
+        inc_s = __builtin_amdgcn_readlane(incl[j], s & 63);
+        full_s = __builtin_amdgcn_readlane(fullc[j], s & 63);
+        ctx_s = __builtin_amdgcn_readlane(ctxv[j], s & 63);
+      }
+    it.seq = __builtin_amdgcn_readfirstlane(s);
+    const int seg = full ? q - (inc_s - full_s) : full_s;
+    it.part0 = seg * m;
+    const int tok_begin = seg * seg_tokens;
+    it.tok_end = full ? tok_begin + seg_tokens : ctx_s;
+    it.c_begin = tok_begin / CT;
+    it.c_end = (it.tok_end + CT - 1) / CT;
+    return it;
+  };
+  // n-th item of this work-group
+  auto position = [&](int nth) { return nth * G + ((nth & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x); };
+
+  // Partial states of two items in flight: the n-th item of this work-group goes to buffer n & 1.
+  __shared__ float sm_m[2][NW][16];
+  __shared__ float sm_l[2][NW][16];
+  __shared__ float sm_acc[2][NW][NR][64];
+  __shared__ int sm_arrived[2];  // wavefronts that have published into the buffer, ever
+
+  if ((int)blockIdx.x >= total_items) return;  // the same for every wavefront of the work-group
+  if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
+  __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
+
+  W wa(p, lane);
+  const int r = wa.r, i = wa.i;
+  Chunk R;
+
+  auto publish = [&](int n) {
+    const int b = n & 1;
+    wa.l = rows_sum(wa.l);
+    if (r == 0) {
+      sm_m[b][wave][i] = wa.m;
+      sm_l[b][wave][i] = wa.l;
+    }
+#pragma unroll
+    for (int e = 0; e < NR; ++e) sm_acc[b][wave][e][lane] = wa.acc_at(e);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0)
+      __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  // Merge the NW published states of the work-group's n-th item, normalise, store this
+  // wavefront's slice of the partial (see the persistent loop kernel for why the wait
+  // always ends and why a buffer is never overwritten while it is read).
+  auto finish = [&](int n, const Item &it) {
+    const int b = n & 1;
+    const int target = NW * ((n >> 1) + 1);
+    for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
+      const int seen = __hip_atomic_load(&sm_arrived[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[b][w][i]);
+    float f[NW];
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float mw = sm_m[b][w][i];
+      f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
+      L += f[w] * sm_l[b][w][i];
+    }
+    float o[SL];
+#pragma unroll
+    for (int e = 0; e < SL; ++e) {
+      float a = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + e][lane];
+      o[e] = a;
+    }
+    if (i < p.group) {
+      const int head = it.kvh * p.group + i;
+      const int64_t slot = ((int64_t)it.seq * p.num_heads + head) * p.max_num_partitions + it.part0;
+      const int d0 = 4 * r * NDT + wave * SL;
+      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, p.out_scale / L);
+      if (r == 0 && wave == 0) {
+        p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
+        p.exp_sums[slot] = L;
+      }
+    }
+  };
+
+  int n = 0;
+  Item cur = decode(position(0));
+  // first chunk of the first item
+  bool armed = cur.c_begin + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  if (armed) {
+    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_begin + wave, col_max);
+    wa.load_q(cur.seq, cur.kvh);
+    wa.issue_k(R, cur.kvh, cur.c_begin + wave, ids);
+    wa.issue_v(R, cur.kvh, cur.c_begin + wave, ids);
+  }
+  uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
+  Item prev = cur;  // the item whose merge is still owed (from the second item on)
+
+  while (true) {
+    const int pn = position(n + 1);
+    const bool has_next = pn < total_items;
+    Item nxt = cur;
+    if (has_next) nxt = decode(pn);
+    const bool next_armed = has_next && nxt.c_begin + wave < nxt.c_end;
+    Ids nxt_ids = {};
+    if (next_armed)
+      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_begin + wave, col_max);
+
+    wa.reset(sink_raw);
+    uint32_t next_sink = W::kNoSink;
+    bool owed = n > 0;
+    if (armed) {
+      const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;
+      int ci = cur.c_begin + wave;
+      Ids nids = wa.fetch_ids(table, ci + NW, col_max);
+      if (ci + NW < cur.c_end) {
+        {  // first chunk of the item, then the merge owed to the previous item
+          const int cn = ci + NW;
+          const auto s = wa.qk(R);
+          wa.issue_k(R, cur.kvh, cn, nids);
+          const auto pb = wa.template soft<false>(R, s, ci, cur.tok_end);
+          wa.pv(R, pb);
+          wa.issue_v(R, cur.kvh, cn, nids);
+          nids = wa.fetch_ids(table, cn + NW, col_max);
+          ci = cn;
+        }
+        if (owed) {
+          finish(n - 1, prev);
+          owed = false;
+        }
+        while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
+          const int cn = ci + NW;
+          const auto s = wa.qk(R);
+          wa.issue_k(R, cur.kvh, cn, nids);
+          const auto pb = wa.template soft<false>(R, s, ci, cur.tok_end);
+          wa.pv(R, pb);
+          wa.issue_v(R, cur.kvh, cn, nids);
+          nids = wa.fetch_ids(table, cn + NW, col_max);
+          ci = cn;
+        }
+      }
+      // last chunk of this wavefront in `cur`: what goes out next belongs to `nxt`
+      const auto s = wa.qk(R);
+      if (next_armed) {
+        wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
+        next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+        wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+      }
+      const auto pb = wa.template soft<true>(R, s, ci, cur.tok_end);
+      wa.pv(R, pb);
+      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+    } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
+      wa.load_q(nxt.seq, nxt.kvh);
+      next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+      wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+    }
+    if (owed) finish(n - 1, prev);
+    publish(n);
+
+    if (!has_next) break;
+    prev = cur;
+    cur = nxt;
+    armed = next_armed;
+    sink_raw = next_sink;
+    ++n;
+  }
+  finish(n, cur);
+}
+
+}  // namespace fa
