@@ -176,6 +176,50 @@ def test_persistent_split_many_items_per_wavefront(oracle):
     torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
 
 
+def test_segment_kernel_partials_lie_a_segment_apart(oracle):
+    """A batch with enough (sequence, kv head) pairs that the split path works in segments of
+    several partitions: the output matches the oracle, and the scratch arrays hold one
+    partial per segment, in the slot of the segment's first partition -- the partials the
+    kernel model gives for a partition size of one segment."""
+    gen = torch.Generator().manual_seed(21)
+    S = 64
+    lens = torch.randint(1, 5000, (S,), generator=gen)
+    lens[5] = 0
+    lens[6] = 4096          # ends exactly on a partition boundary
+    w = W.make_config(4, num_seqs=S, pool_blocks=S * 320, lens=lens.tolist())   # bf16 queries, E5M2 pools, G = 8
+    w.sinks = torch.linspace(-1, 3, w.num_heads).to(w.query.dtype)
+    from flash_attention_factory_amd import runner
+    wd = w.to(_dev())
+    bufs = runner.alloc_buffers(wd)
+    for t in (bufs.exp_sums, bufs.max_logits, bufs.tmp_out):
+        t.fill_(float("nan"))
+    runner.run_workload(wd, "fp8_reduce", bufs)
+    torch.cuda.synchronize()
+    out = bufs.out.cpu()
+    ref = call_oracle(oracle.attention_ref, w)
+    live = lens > 0
+    torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
+    # which slots were written: 0, m, 2m, ...
+    es = bufs.exp_sums.cpu()
+    longest = int(lens.argmax())
+    written = (~torch.isnan(es[longest, 0])).nonzero().flatten().tolist()
+    assert written[0] == 0 and len(written) >= 2
+    m = written[1]
+    assert m >= 2, "this batch is meant to be cut into multi-partition segments"
+    P = w.partition_size
+    for s in range(S):
+        nseg = -(-int(lens[s]) // (m * P))
+        want = [j * m for j in range(nseg)]
+        assert (~torch.isnan(es[s, 0])).nonzero().flatten().tolist() == want, s
+    NP = bufs.exp_sums.shape[2]
+    mes, mml, mtmp = call_oracle(oracle.kernel_partition, w, partition_size=m * P, max_num_partitions=NP)
+    for s in range(S):
+        for j in range(-(-int(lens[s]) // (m * P))):
+            torch.testing.assert_close(bufs.max_logits[s, :, j * m].cpu(), mml[s, :, j], atol=1e-3, rtol=1e-4)
+            torch.testing.assert_close(es[s, :, j * m], mes[s, :, j], atol=1e-3, rtol=2e-3)
+            torch.testing.assert_close(bufs.tmp_out[s, :, j * m].cpu(), mtmp[s, :, j], atol=1e-2, rtol=1e-2)
+
+
 @pytest.mark.parametrize("batch,heads", [(300, 16), (128, 32)])
 def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
     """From 4096 (sequence, head) pairs on the reduce kernel runs one wavefront per pair;
