@@ -16,7 +16,6 @@
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
 #include "paged_attention_loop_persistent_kernel.h"
-#include "paged_attention_persistent_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
 #include "paged_attention_segment_kernel.h"

@@ -26,10 +26,10 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   const PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache,
                                         value_cache, block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
-  // kernel 1.  Persistent form when the batch fits it: as many single-wavefront
-  // work-groups as the GPU keeps resident walk the list of live partitions.  Otherwise
-  // one work-group per (kv head, partition slot, sequence); slots past a sequence's
-  // length return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
+  // kernel 1.  Segment form when the batch fits it: as many multi-wavefront work-groups as
+  // the GPU keeps resident share out segments of several partitions.  Otherwise one
+  // work-group per (kv head, partition slot, sequence); slots past a sequence's length
+  // return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
   int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
   if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
       (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
@@ -43,15 +43,6 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
         (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
     segment_groups = (int)std::min<int64_t>(resident, max_items);
     FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
-  } else if (kUsePersistentSplit && shape.num_seqs <= kPersistentMaxSeqs && shape.num_pool_blocks > 0) {
-    auto kernel = paged_attn_split_persistent_kernel<HEAD_SIZE, QT, KV8, Pipeline<KV8>::occ,
-                                                     Pipeline<KV8>::tiles_per_chunk, SplitOrder<KV8>::value>;
-    int resident = 0;
-    FA_HIP_CHECK(resident_groups(kernel, 64, &resident));
-    const int64_t max_items =
-        (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
-    const dim3 grid((unsigned)std::min<int64_t>(resident, max_items));
-    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(64), 0, p));
   } else {
     const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(

@@ -39,7 +39,7 @@ struct WavesPerGroup {
 // Per cache type: wavefronts per SIMD the register allocator must fit (4 SIMDs per CU),
 // tiles per chunk, and whether K/V loads are marked non-temporal (the bytes are read once
 // per launch).  Non-temporal loads measured +4..5 % on 16-bit caches in both paths and
-// +10 % on the FP8 loop path, but -3 % on the FP8 split path.
+// +10 % on the FP8 loop path, but -3 % on the grid form of the FP8 split path.
 #ifndef FA_OCC
 #define FA_OCC 3
 #endif
@@ -70,25 +70,6 @@ struct Pipeline {
 };
 
 // ---- persistent kernels (batches of up to 128 / 256 sequences) -------------------------
-// Split path: resident single-wavefront work-groups walk the live partitions.
-#ifndef FA_PERSISTENT_SPLIT
-#define FA_PERSISTENT_SPLIT 1
-#endif
-constexpr bool kUsePersistentSplit = FA_PERSISTENT_SPLIT != 0;
-// Item order of the persistent split kernel (0: kv head fastest, interleaved over all
-// work-groups; 1: partition fastest, one contiguous range of items per XCD).  Measured:
-// order 1 is 2 % faster with 16-bit caches, order 0 is 1 % faster with FP8 caches.
-#ifndef FA_SPLIT_ORDER
-#define FA_SPLIT_ORDER 1
-#endif
-#ifndef FA_SPLIT_ORDER_FP8
-#define FA_SPLIT_ORDER_FP8 0
-#endif
-template <bool kKV8>
-struct SplitOrder {
-  static constexpr int value = kKV8 ? FA_SPLIT_ORDER_FP8 : FA_SPLIT_ORDER;
-};
-
 // Split path, segment form: multi-wavefront work-groups take segments of several partitions
 // and write one partial per segment (paged_attention_segment_kernel.h).
 #ifndef FA_SPLIT_SEGMENT
@@ -111,8 +92,8 @@ struct SegmentSplit {
   static constexpr bool use = (kKV8 ? FA_SPLIT_SEGMENT_FP8 : FA_SPLIT_SEGMENT) != 0;
   static constexpr int waves = FA_SEGMENT_WAVES;
   static constexpr int occ = FA_SEGMENT_OCC;
-  // non-temporal K/V loads: +5 % here for both cache types (long streaming runs per
-  // wavefront, as in the loop kernels)
+  // non-temporal K/V loads, as in the loop kernels (long streaming runs per wavefront):
+  // measured +5 % with an FP8 cache
   static constexpr bool stream_loads = FA_SEGMENT_STREAM_LOADS != 0;
 };
 
