@@ -8,11 +8,15 @@
 //
 // One work-group of one or four wavefronts per (sequence, head).  The kernel is a chain
 // of dependent memory round trips, so it is built to have as few of them as possible:
-// wavefront w owns partitions w, w+NW, w+2NW, ... and requests up to 16 of their tmp_out
+// wavefront w owns partitions w, w+NW, w+2NW, ... and requests up to 16 (4) of their tmp_out
 // rows (one coalesced 512-byte row per load) together with the partition scalars, before
 // anything is waited for; the weights are applied when both have arrived; with four
 // wavefronts the partial sums meet in LDS.  Lane j owns D/64 consecutive output elements.
 #pragma once
+
+#ifndef FA_REDUCE_SEGMENT_ROWS
+#define FA_REDUCE_SEGMENT_ROWS 4
+#endif
 
 #include "paged_attention_segment_policy.h"
 #include "paged_attention_utils.h"
@@ -36,7 +40,11 @@ struct ReduceParams {
                            // segment's first slot); 0: one partial per partition
 };
 
-constexpr int kReduceRowsInFlight = 16;  // per wavefront and batch
+// Rows requested per wavefront and batch: 16 when every partition has a partial (dozens per
+// sequence); 4 after the segment kernel, which leaves a handful per sequence -- the smaller
+// register set then lets twice as many work-groups stay resident.
+template <bool SEGMENTS>
+constexpr int reduce_rows_in_flight() { return SEGMENTS ? FA_REDUCE_SEGMENT_ROWS : 16; }
 
 // kReduceWaves wavefronts per (sequence, head): 4 when there are few (sequence, head)
 // pairs -- the launch is then short of parallelism and each pair's rows should be in
@@ -45,7 +53,7 @@ constexpr int kReduceRowsInFlight = 16;  // per wavefront and batch
 template <int D, typename QT, int kReduceWaves, bool SEGMENTS = false>
 __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
   constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
-  constexpr int R = kReduceRowsInFlight;
+  constexpr int R = reduce_rows_in_flight<SEGMENTS>();
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int head = blockIdx.x;
