@@ -118,7 +118,11 @@ int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_ca
                                 const fa_paged_attention_shape *shape,
                                 const fa_paged_attention_options *options);
 
-/* Split-context kernel followed by the reduce kernel. */
+/* Split-context kernel followed by the reduce kernel.  exp_sums, max_logits and tmp_out are
+ * scratch the two kernels hand partial softmax states through; every slot either holds what
+ * upstream stores there for its partition -- or nothing: for batches with many
+ * (sequence, kv head) pairs one partial covers several consecutive partitions and sits in
+ * the slot of the first, the slots in between staying untouched.  Only `out` is a result. */
 int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
                                   const void *value_cache, const int32_t *block_tables,
                                   const int32_t *context_lens, float scale,
