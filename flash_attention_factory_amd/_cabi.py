@@ -35,6 +35,10 @@ EXPORTS = (
 
 FA_KV_CACHE_16BIT = 0
 FA_KV_CACHE_E5M2 = 1
+FA_KV_CACHE_E4M3 = 2
+
+FA_FP8_E5M2 = 0
+FA_FP8_E4M3 = 1
 
 
 class Shape(ctypes.Structure):
@@ -64,7 +68,7 @@ class Options(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("elapsed_us", ctypes.POINTER(ctypes.c_float)),
         ("validate_only", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("kv_fp8_format", ctypes.c_int32),
     ]
 
 

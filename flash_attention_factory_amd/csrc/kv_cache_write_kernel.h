@@ -43,14 +43,6 @@ struct KvWriteParams {
   int64_t src_head_bytes;
 };
 
-// fp32 -> E5M2 byte exactly as the tensor cast does it, in software: round to nearest
-// even, 65536 and beyond (infinity included) to infinity, NaN to 0x7f with its sign.
-// Only NaN ever comes here; everything else goes through the conversion instruction.
-__device__ __forceinline__ uint32_t e5m2_nan_or_keep(float f, uint32_t converted) {
-  const uint32_t x = __builtin_bit_cast(uint32_t, f);
-  return (x & 0x7fffffffu) > 0x7f800000u ? (0x7fu | ((x >> 24) & 0x80u)) : converted;
-}
-
 template <typename ST>
 __device__ __forceinline__ float f32_from_half_of(uint32_t w, int hi) {
   if constexpr (std::is_same<ST, BF16>::value) {
@@ -61,13 +53,16 @@ __device__ __forceinline__ float f32_from_half_of(uint32_t w, int hi) {
   }
 }
 
-// 8 source elements (4 dwords) -> 8 E5M2 bytes (2 dwords).  v_cvt_pk_bf8_f32 rounds two
-// fp32 values to nearest even, sends what lies beyond the E5M2 range to infinity and
-// handles subnormals -- checked against the tensor cast on every fp16 and bf16 input --
-// but it has its own NaN pattern, so NaN bytes (exponent 31, mantissa not 0) are spotted
-// in the result and rewritten to the cast's 0x7f | sign.
-template <typename ST, bool SCALED>
-__device__ __forceinline__ u32x2 e5m2_from_row_piece(u32x4 src, float mul) {
+// 8 source elements (4 dwords) -> 8 FP8 bytes (2 dwords).
+// E5M2: v_cvt_pk_bf8_f32 rounds two fp32 values to nearest even, sends what lies beyond the
+// range to infinity and handles subnormals -- checked against the tensor cast on every fp16
+// and bf16 input -- but it has its own NaN pattern, so NaN bytes (exponent 31, mantissa not
+// 0) are spotted in the result and rewritten to the cast's 0x7f | sign.
+// E4M3: v_cvt_pk_fp8_f32 likewise; the format has no infinity and the cast turns everything
+// that rounds beyond 448 (480 and above, NaN included) into NaN, 0x7f | sign, which is
+// decided here from the inputs, whatever the instruction does with them.
+template <typename ST, int KVF, bool SCALED>
+__device__ __forceinline__ u32x2 fp8_from_row_piece(u32x4 src, float mul) {
   float f[8];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -81,15 +76,31 @@ __device__ __forceinline__ u32x2 e5m2_from_row_piece(u32x4 src, float mul) {
   u32x2 out;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    int w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h], f[4 * h + 1], 0, false);
-    w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h + 2], f[4 * h + 3], w, true);
-    uint32_t u = (uint32_t)w;
-    // any byte with magnitude bits above 0x7c is a NaN
-    if ((((u & 0x7f7f7f7fu) + 0x03030303u) & 0x80808080u) != 0) {
+    uint32_t u;
+    bool fix;
+    if constexpr (KVF == kKvE4M3) {
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h], f[4 * h + 1], 0, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h + 2], f[4 * h + 3], w, true);
+      u = (uint32_t)w;
+      // 480 and above, infinity and NaN all have magnitude bits >= those of 480.0f
+      uint32_t big = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) big = max(big, __builtin_bit_cast(uint32_t, f[4 * h + e]) & 0x7fffffffu);
+      fix = big >= 0x43f00000u;
+    } else {
+      int w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h], f[4 * h + 1], 0, false);
+      w = __builtin_amdgcn_cvt_pk_bf8_f32(f[4 * h + 2], f[4 * h + 3], w, true);
+      u = (uint32_t)w;
+      // any byte with magnitude bits above 0x7c is a NaN
+      fix = (((u & 0x7f7f7f7fu) + 0x03030303u) & 0x80808080u) != 0;
+    }
+    if (fix) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const uint32_t b = e5m2_nan_or_keep(f[4 * h + e], (u >> (8 * e)) & 0xffu);
-        u = (u & ~(0xffu << (8 * e))) | (b << (8 * e));
+        const uint32_t x = __builtin_bit_cast(uint32_t, f[4 * h + e]);
+        const uint32_t mag = x & 0x7fffffffu;
+        const bool special = KVF == kKvE4M3 ? mag >= 0x43f00000u /* 480.0f */ : mag > 0x7f800000u /* NaN */;
+        if (special) u = (u & ~(0xffu << (8 * e))) | ((0x7fu | ((x >> 24) & 0x80u)) << (8 * e));
       }
     }
     out[h] = u;
@@ -97,8 +108,9 @@ __device__ __forceinline__ u32x2 e5m2_from_row_piece(u32x4 src, float mul) {
   return out;
 }
 
-template <typename ST, bool KV8, bool SCALED>
+template <typename ST, int KVF, bool SCALED>
 __global__ void __launch_bounds__(256) kv_cache_write_kernel(const KvWriteParams p) {
+  constexpr bool KV8 = KVF != kKv16;
   const int ppt = p.pieces_per_token;
   // place inside the group of tokens a work-group covers per step
   const int local_token = (int)threadIdx.x / ppt;  // 0 when a token has more pieces than threads
@@ -124,8 +136,8 @@ __global__ void __launch_bounds__(256) kv_cache_write_kernel(const KvWriteParams
       const uint32_t row = s - block * (uint32_t)p.block_size;
       const int64_t dst = (int64_t)block * p.kv_block_bytes + (int64_t)row * p.kv_token_bytes + dst_off;
       if constexpr (KV8) {
-        *reinterpret_cast<u32x2 *>(p.key_cache + dst) = e5m2_from_row_piece<ST, SCALED>(k, p.inv_scale);
-        *reinterpret_cast<u32x2 *>(p.value_cache + dst) = e5m2_from_row_piece<ST, SCALED>(v, p.inv_scale);
+        *reinterpret_cast<u32x2 *>(p.key_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(k, p.inv_scale);
+        *reinterpret_cast<u32x2 *>(p.value_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(v, p.inv_scale);
       } else {
         *reinterpret_cast<u32x4 *>(p.key_cache + dst) = k;
         *reinterpret_cast<u32x4 *>(p.value_cache + dst) = v;

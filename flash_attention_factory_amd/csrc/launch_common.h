@@ -54,6 +54,7 @@ struct Resolved {
   int32_t partition_size;
   int32_t kv_elem_bytes;
   float fp8_scale;
+  bool e4m3;  // FP8 entries: the caches hold E4M3 bytes, not E5M2
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -121,6 +122,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
       (int64_t)s->max_blocks_per_seq * s->block_size < (int64_t)max_context_len)
     return fail(FA_ERR_BAD_SHAPE, "max_context_len %d does not fit %d blocks of %d tokens", max_context_len,
                 s->max_blocks_per_seq, s->block_size);
+  if (kv8 && o && o->kv_fp8_format != FA_FP8_E5M2 && o->kv_fp8_format != FA_FP8_E4M3)
+    return fail(FA_ERR_UNSUPPORTED_DTYPE, "kv_fp8_format %d is neither E5M2 (0) nor E4M3 (1)", o->kv_fp8_format);
+  r->e4m3 = kv8 && o && o->kv_fp8_format == FA_FP8_E4M3;
   r->fp8_scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
   r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   r->elapsed_us = o ? o->elapsed_us : nullptr;

@@ -14,13 +14,14 @@
 namespace fa {
 
 // One launch, grid (kv heads, 1, sequences), NW wavefronts per work-group.
-// KV8 selects the E5M2 cache form (used by launch_kernels_fp8_loop.h).
-template <int HEAD_SIZE, typename QT, bool KV8>
+// KVF selects the cache format: 16-bit, or E5M2 / E4M3 bytes (launch_kernels_fp8_loop.h).
+template <int HEAD_SIZE, typename QT, int KVF>
 inline fa_status launch_paged_attn_loop(void *out, const void *query, const void *key_cache,
                                         const void *value_cache, const int32_t *block_tables,
                                         const int32_t *context_lens, float scale,
                                         int32_t /*max_context_len: validation only*/,
                                         const fa_paged_attention_shape &shape, const Resolved &r) {
+  constexpr bool KV8 = KVF != kKv16;
   constexpr int NW = WavesPerGroup<false>::value;
   const PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
                                         block_tables, context_lens, scale, shape, r);
@@ -32,7 +33,7 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
     // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
     // sequences first, with the next item's first loads issued before each merge.
     constexpr int PW = PersistentLoop<KV8>::waves;
-    auto kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KV8, PW, PersistentLoop<KV8>::occ,
+    auto kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
                                                     Pipeline<KV8>::tiles_per_chunk>;
     int resident = 0;
     FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
@@ -41,7 +42,7 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   } else {
     const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KV8, false, NW, Pipeline<KV8>::occ,
+        paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
                           Pipeline<KV8>::tiles_per_chunk>,
         grid, dim3(NW * 64), 0, p));
   }
@@ -64,8 +65,19 @@ inline fa_status dispatch_paged_attention_loop_any(void *out, const void *query,
   if (st != FA_OK || r.validate_only) return st;
   const bool bf16 = shape->q_dtype == FA_DTYPE_BF16;
 #define FA_LOOP_CASE(HS, QT)                                                                      \
-  return launch_paged_attn_loop<HS, QT, KV8>(out, query, key_cache, value_cache, block_tables,    \
-                                             context_lens, scale, max_context_len, *shape, r)
+  do {                                                                                            \
+    if (!KV8)                                                                                     \
+      return launch_paged_attn_loop<HS, QT, kKv16>(out, query, key_cache, value_cache,            \
+                                                   block_tables, context_lens, scale,             \
+                                                   max_context_len, *shape, r);                   \
+    if (r.e4m3)                                                                                   \
+      return launch_paged_attn_loop<HS, QT, kKvE4M3>(out, query, key_cache, value_cache,          \
+                                                     block_tables, context_lens, scale,           \
+                                                     max_context_len, *shape, r);                 \
+    return launch_paged_attn_loop<HS, QT, kKvE5M2>(out, query, key_cache, value_cache,            \
+                                                   block_tables, context_lens, scale,             \
+                                                   max_context_len, *shape, r);                   \
+  } while (0)
   if (shape->head_size == 128) {
     if (bf16) FA_LOOP_CASE(128, BF16);
     FA_LOOP_CASE(128, F16);

@@ -15,13 +15,14 @@
 
 namespace fa {
 
-template <int HEAD_SIZE, typename QT, bool KV8>
+template <int HEAD_SIZE, typename QT, int KVF>
 inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *key_cache,
                                       const void *value_cache, const int32_t *block_tables,
                                       const int32_t *context_lens, float scale,
                                       int32_t /*max_context_len: validation only*/,
                                       float *exp_sums, float *max_logits, float *tmp_out,
                                       const fa_paged_attention_shape &shape, const Resolved &r) {
+  constexpr bool KV8 = KVF != kKv16;
   constexpr int NW = WavesPerGroup<true>::value;
   const PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache,
                                         value_cache, block_tables, context_lens, scale, shape, r);
@@ -35,7 +36,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
       (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
     // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
     constexpr int SW = SegmentSplit<KV8>::waves;
-    auto kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KV8, SW, SegmentSplit<KV8>::occ,
+    auto kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                             Pipeline<KV8>::tiles_per_chunk>;
     int resident = 0;
     FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
@@ -46,7 +47,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   } else {
     const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KV8, true, NW, Pipeline<KV8>::occ,
+        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
                           Pipeline<KV8>::tiles_per_chunk>,
         grid, dim3(NW * 64), 0, p));
   }
@@ -97,9 +98,22 @@ inline fa_status dispatch_paged_attention_any(void *out, const void *query, cons
   if (st != FA_OK || r.validate_only) return st;
   const bool bf16 = shape->q_dtype == FA_DTYPE_BF16;
 #define FA_V2_CASE(HS, QT)                                                                       \
-  return launch_paged_attn_v2<HS, QT, KV8>(out, query, key_cache, value_cache, block_tables,     \
-                                           context_lens, scale, max_context_len, exp_sums,       \
-                                           max_logits, tmp_out, *shape, r)
+  do {                                                                                           \
+    if (!KV8)                                                                                    \
+      return launch_paged_attn_v2<HS, QT, kKv16>(out, query, key_cache, value_cache,             \
+                                                 block_tables, context_lens, scale,              \
+                                                 max_context_len, exp_sums, max_logits, tmp_out, \
+                                                 *shape, r);                                     \
+    if (r.e4m3)                                                                                  \
+      return launch_paged_attn_v2<HS, QT, kKvE4M3>(out, query, key_cache, value_cache,           \
+                                                   block_tables, context_lens, scale,            \
+                                                   max_context_len, exp_sums, max_logits,        \
+                                                   tmp_out, *shape, r);                          \
+    return launch_paged_attn_v2<HS, QT, kKvE5M2>(out, query, key_cache, value_cache,             \
+                                                 block_tables, context_lens, scale,              \
+                                                 max_context_len, exp_sums, max_logits, tmp_out, \
+                                                 *shape, r);                                     \
+  } while (0)
   if (shape->head_size == 128) {
     if (bf16) FA_V2_CASE(128, BF16);
     FA_V2_CASE(128, F16);

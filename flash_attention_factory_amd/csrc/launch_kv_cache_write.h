@@ -23,13 +23,14 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
     return fail(FA_ERR_NULL_POINTER, "key, value, key_cache, value_cache and slot_mapping must all be non-NULL");
   if (s->src_dtype != FA_DTYPE_F16 && s->src_dtype != FA_DTYPE_BF16)
     return fail(FA_ERR_UNSUPPORTED_DTYPE, "src_dtype %d is neither fp16 (0) nor bf16 (1)", s->src_dtype);
-  if (s->cache_dtype != FA_KV_CACHE_16BIT && s->cache_dtype != FA_KV_CACHE_E5M2)
-    return fail(FA_ERR_UNSUPPORTED_DTYPE, "cache_dtype %d is neither 16-bit (0) nor E5M2 (1)", s->cache_dtype);
+  if (s->cache_dtype != FA_KV_CACHE_16BIT && s->cache_dtype != FA_KV_CACHE_E5M2 && s->cache_dtype != FA_KV_CACHE_E4M3)
+    return fail(FA_ERR_UNSUPPORTED_DTYPE, "cache_dtype %d is none of 16-bit (0), E5M2 (1), E4M3 (2)", s->cache_dtype);
   if (s->num_tokens < 0 || s->num_kv_heads <= 0 || s->block_size <= 0 || s->num_pool_blocks <= 0)
     return fail(FA_ERR_BAD_SHAPE, "num_tokens must be >= 0; num_kv_heads, block_size and num_pool_blocks positive");
   if (s->head_size <= 0 || s->head_size % 8)
     return fail(FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE, "head_size %d must be a positive multiple of 8", s->head_size);
-  const bool kv8 = s->cache_dtype == FA_KV_CACHE_E5M2;
+  const bool kv8 = s->cache_dtype != FA_KV_CACHE_16BIT;
+  const bool e4m3 = s->cache_dtype == FA_KV_CACHE_E4M3;
   const int64_t eb = kv8 ? 1 : 2;
   const int64_t src_head = s->src_head_stride > 0 ? s->src_head_stride : s->head_size;
   const int64_t src_token = s->src_token_stride > 0 ? s->src_token_stride : src_head * s->num_kv_heads;
@@ -84,15 +85,17 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   const dim3 grid((unsigned)std::min<int64_t>(groups_needed, 0x7fffffff)), block(256);
   const bool bf16 = s->src_dtype == FA_DTYPE_BF16;
   const bool scaled = scale != 1.0f;
+#define FA_KVW_LAUNCH(ST, KVF, SC) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<ST, KVF, SC>, grid, block, 0, p))
   if (!kv8) {  // a 16-bit pool takes bit copies whatever the 16-bit type
-    FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, false, false>, grid, block, 0, p));
-  } else if (bf16) {
-    if (scaled) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<BF16, true, true>, grid, block, 0, p));
-    else FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<BF16, true, false>, grid, block, 0, p));
+    FA_KVW_LAUNCH(F16, kKv16, false);
+  } else if (e4m3) {
+    if (bf16) { if (scaled) FA_KVW_LAUNCH(BF16, kKvE4M3, true); else FA_KVW_LAUNCH(BF16, kKvE4M3, false); }
+    else { if (scaled) FA_KVW_LAUNCH(F16, kKvE4M3, true); else FA_KVW_LAUNCH(F16, kKvE4M3, false); }
   } else {
-    if (scaled) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, true>, grid, block, 0, p));
-    else FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<F16, true, false>, grid, block, 0, p));
+    if (bf16) { if (scaled) FA_KVW_LAUNCH(BF16, kKvE5M2, true); else FA_KVW_LAUNCH(BF16, kKvE5M2, false); }
+    else { if (scaled) FA_KVW_LAUNCH(F16, kKvE5M2, true); else FA_KVW_LAUNCH(F16, kKvE5M2, false); }
   }
+#undef FA_KVW_LAUNCH
   if (o && o->elapsed_us) FA_HIP_CHECK(timer.read(0, &o->elapsed_us[0]));
   return FA_OK;
 }

@@ -89,10 +89,10 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   }
 }
 
-template <int D, typename QT, bool KV8, bool PART, int NW, int OCC, int TPC>
+template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KV8, TPC, PART ? Pipeline<KV8>::stream_loads_split : Pipeline<KV8>::stream_loads_loop>;
+  using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;

@@ -28,10 +28,10 @@ constexpr int kLoopPersistentMaxContext = 1 << 24;  // lengths are packed into 2
 // item -- it only turns a would-be hang into a wrong answer that the tests catch.
 constexpr int kLoopPersistentSpinLimit = 1 << 24;
 
-template <int D, typename QT, bool KV8, int NW, int OCC, int TPC>
+template <int D, typename QT, int KVF, int NW, int OCC, int TPC>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KV8, TPC, Pipeline<KV8>::stream_loads_loop>;
+  using W = WaveAttn<D, QT, KVF, TPC, Pipeline<(KVF != 0)>::stream_loads_loop>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;

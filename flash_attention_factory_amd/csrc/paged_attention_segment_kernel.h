@@ -26,10 +26,10 @@
 
 namespace fa {
 
-template <int D, typename QT, bool KV8, int NW, int OCC, int TPC>
+template <int D, typename QT, int KVF, int NW, int OCC, int TPC>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_segment_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KV8, TPC, SegmentSplit<KV8>::stream_loads>;
+  using W = WaveAttn<D, QT, KVF, TPC, SegmentSplit<(KVF != 0)>::stream_loads>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;

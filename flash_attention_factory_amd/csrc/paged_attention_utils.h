@@ -11,6 +11,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace fa {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -103,6 +105,41 @@ __device__ __forceinline__ uint32_t e5m2_adjacent_pair<BF16>(uint32_t w, int hal
   bf16x2 v = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, false)
                        : __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, true);
   return __builtin_bit_cast(uint32_t, v);
+}
+
+// FP8 cache formats.  kKvE5M2: 1-5-2, binary16 cut to its top byte.  kKvE4M3: 1-4-3 "fn"
+// (bias 7, no infinities, 0x7f / 0xff NaN), decoded by the CDNA4 conversion instructions;
+// both decode exactly into fp16 and bf16.
+constexpr int kKv16 = 0, kKvE5M2 = 1, kKvE4M3 = 2;
+
+template <int KVF, typename QT>
+__device__ __forceinline__ uint32_t fp8_pair(uint32_t lo_byte, uint32_t hi_byte) {
+  if constexpr (KVF == kKvE4M3) {
+    const uint32_t two = lo_byte | (hi_byte << 8);
+    if constexpr (std::is_same<QT, BF16>::value) {
+      return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(two, 1.0f, false));
+    } else {
+      return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(two, 1.0f, false));
+    }
+  } else {
+    return e5m2_pair<QT>(lo_byte, hi_byte);
+  }
+}
+template <int KVF, typename QT>
+__device__ __forceinline__ uint32_t fp8_adjacent_pair(uint32_t w, int half) {
+  if constexpr (KVF == kKvE4M3) {
+    if constexpr (std::is_same<QT, BF16>::value) {
+      const bf16x2 v = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false)
+                                 : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+      return __builtin_bit_cast(uint32_t, v);
+    } else {
+      const f16x2 v = half == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false)
+                                : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+      return __builtin_bit_cast(uint32_t, v);
+    }
+  } else {
+    return e5m2_adjacent_pair<QT>(w, half);
+  }
 }
 
 // Reductions over the four 16-lane rows of a wavefront (lanes i, i+16, i+32, i+48).

@@ -1,6 +1,6 @@
 // One wavefront's share of paged-attention decode on gfx950: operand loads, the two
 // MFMA products and the online softmax between them.  The grid kernel and the
-// persistent kernel are both built from this.
+// persistent kernels are all built from this.
 //
 // Per chunk of TPC 16-token tiles (the query group's G <= 16 heads are the 16 MFMA columns):
 //   S^T[token, head] = K[token, :] . Q^T[:, head]      per tile: D/32 MFMA 16x16x32
@@ -52,8 +52,10 @@ struct PagedAttnParams {
 
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
-template <int D, typename QT, bool KV8, int TPC, bool STREAM>
+// KVF: cache format, kKv16 (elements of the query type), kKvE5M2 or kKvE4M3 (bytes).
+template <int D, typename QT, int KVF, int TPC, bool STREAM>
 struct WaveAttn {
+  static constexpr bool KV8 = KVF != kKv16;
   static_assert(TPC == 2 || TPC == 4, "a chunk is one or two 32-token P.V steps");
   static constexpr int ROWB = D * (KV8 ? 1 : 2);  // bytes per token row
   static constexpr int KL = ROWB / 64;            // 16-byte K loads per lane and tile
@@ -177,10 +179,10 @@ struct WaveAttn {
       const u32x4 src = R.k[tile][c >> 1];
       const int h = c & 1;
       u32x4 o;
-      o[0] = e5m2_adjacent_pair<QT>(src[2 * h], 0);
-      o[1] = e5m2_adjacent_pair<QT>(src[2 * h], 1);
-      o[2] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 0);
-      o[3] = e5m2_adjacent_pair<QT>(src[2 * h + 1], 1);
+      o[0] = fp8_adjacent_pair<KVF, QT>(src[2 * h], 0);
+      o[1] = fp8_adjacent_pair<KVF, QT>(src[2 * h], 1);
+      o[2] = fp8_adjacent_pair<KVF, QT>(src[2 * h + 1], 0);
+      o[3] = fp8_adjacent_pair<KVF, QT>(src[2 * h + 1], 1);
       return o;
     }
   }
@@ -199,7 +201,7 @@ struct WaveAttn {
       } else {
         const uint32_t y = (R.v[e0][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
         const uint32_t x = (R.v[e0 + 1][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
-        o[c] = e5m2_pair<QT>(y, x);
+        o[c] = fp8_pair<KVF, QT>(y, x);
       }
     }
     return o;

@@ -53,7 +53,7 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
                                         "block_tables and context_lens must be int32")
-    want_kv = (torch.float8_e5m2, torch.uint8) if fp8 else (query.dtype,)
+    want_kv = (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8) if fp8 else (query.dtype,)
     if key_cache.dtype not in want_kv or value_cache.dtype != key_cache.dtype:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
                                         f"key/value cache dtype {key_cache.dtype} not in {want_kv}")
@@ -85,6 +85,8 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     op.alibi_slopes = alibi_slopes.data_ptr() if alibi_slopes is not None else None
     op.softcap = softcap
     op.fp8_scale = fp8_scale
+    # bytes are E5M2 as upstream fixes them (paged_attention_fp8_loop.cpp:43) unless the tensor says E4M3
+    op.kv_fp8_format = _cabi.FA_FP8_E4M3 if key_cache.dtype == torch.float8_e4m3fn else _cabi.FA_FP8_E5M2
     op.stream = torch.cuda.current_stream(query.device).cuda_stream
     op.elapsed_us = ctypes.cast(elapsed, ctypes.POINTER(ctypes.c_float)) if timed else None
     fn = getattr(L, entry)

@@ -1,5 +1,5 @@
 """``kv_cache_write.run``: scatter new K/V token rows into the paged pools the decode
-kernels read, rounding to FP8 E5M2 when the pools hold bytes.
+kernels read, rounding to FP8 (E5M2, or E4M3 for ``torch.float8_e4m3fn`` pools) when the pools hold bytes.
 
 Upstream has no extension module for this step; its tests build the pools with tensor
 casts (test_paged_fp8cache.py:171-203: ``k_cache_paged.to(torch.float8_e5m2)``).  The
@@ -31,10 +31,10 @@ def run(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_c
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
                                         "key and value must be [tokens, kv_heads, head_size] with equal "
                                         "strides and a contiguous last dimension")
-    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.uint8)
+    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8)
     if (not fp8 and key_cache.dtype != key.dtype) or value_cache.dtype != key_cache.dtype:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,
-                                        f"cache dtype {key_cache.dtype} is neither the source dtype nor E5M2")
+                                        f"cache dtype {key_cache.dtype} is neither the source dtype nor an FP8 format")
     if key_cache.dim() != 4 or key_cache.stride(3) != 1 or value_cache.stride() != key_cache.stride() \
             or key_cache.size(2) != key.size(1) or key_cache.size(3) != key.size(2):
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
@@ -49,7 +49,8 @@ def run(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_c
         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
     sh.src_token_stride, sh.src_head_stride = key.stride(0), key.stride(1)
     sh.src_dtype = _cabi.FA_DTYPE_BF16 if key.dtype == torch.bfloat16 else _cabi.FA_DTYPE_F16
-    sh.cache_dtype = _cabi.FA_KV_CACHE_E5M2 if fp8 else _cabi.FA_KV_CACHE_16BIT
+    sh.cache_dtype = _cabi.FA_KV_CACHE_16BIT if not fp8 else (
+        _cabi.FA_KV_CACHE_E4M3 if key_cache.dtype == torch.float8_e4m3fn else _cabi.FA_KV_CACHE_E5M2)
     sh.num_pool_blocks = key_cache.size(0)
     elapsed = (ctypes.c_float * 2)(0.0, 0.0)
     op = _cabi.Options()

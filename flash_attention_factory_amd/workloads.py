@@ -31,7 +31,7 @@ TOKEN_MAJOR = "token_major"  # [num_blocks, block_size, num_kv_heads, head_size]
 class Workload:
     name: str
     query: torch.Tensor            # [S, H, D] fp16 / bf16
-    key_cache: torch.Tensor        # 4-D pool, 16-bit or float8_e5m2
+    key_cache: torch.Tensor        # 4-D pool, 16-bit, float8_e5m2 or float8_e4m3fn
     value_cache: torch.Tensor
     block_tables: torch.Tensor     # [S, MB] int32
     context_lens: torch.Tensor     # [S] int32
@@ -46,7 +46,7 @@ class Workload:
 
     @property
     def is_fp8(self) -> bool:
-        return self.key_cache.dtype == torch.float8_e5m2
+        return self.key_cache.dtype in (torch.float8_e5m2, torch.float8_e4m3fn)
 
     @property
     def num_seqs(self) -> int:
@@ -168,13 +168,15 @@ def _randn16_on(shape, device, seed, dtype):
 
 def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs: Optional[int] = None,
                 pool_blocks: Optional[int] = None, device="cpu", pools_on_device: bool = False,
-                lens=None) -> Workload:
+                lens=None, fp8_dtype=torch.float8_e5m2) -> Workload:
     """One of the five measured configurations.  ``num_seqs``/``pool_blocks`` shrink
     a configuration for CPU-sized parity runs without changing anything else.
     ``pools_on_device`` draws the two KV pools with the target device's own generator
     (same distribution, different bits) -- for throughput runs, where drawing a
     gigabyte of normals on the host would dominate the run.  ``lens`` replaces the
-    drawn context lengths (the block tables are dealt for the lengths in force)."""
+    drawn context lengths (the block tables are dealt for the lengths in force).
+    ``fp8_dtype`` is the byte format of an FP8 configuration's pools: E5M2 as upstream,
+    or ``torch.float8_e4m3fn``."""
     c = _CONFIGS[index]
     S = num_seqs or c["S"]
     H, Hk, D, B = c["H"], c["Hk"], c["D"], c["B"]
@@ -193,8 +195,8 @@ def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs
         v = _randn16(shape, gen, kv16)
     if c["fp8"]:
         # cast of fp16 N(0,1) samples, as test_paged_fp8cache.py:201-203 does
-        k = k.to(torch.float8_e5m2)
-        v = v.to(torch.float8_e5m2)
+        k = k.to(fp8_dtype)
+        v = v.to(fp8_dtype)
     perm = torch.randperm(NB, generator=gen, dtype=torch.int64).to(torch.int32)
     drawn = _draw_lens(c["lens"], S, gen)
     lens = drawn if lens is None else torch.as_tensor(lens, dtype=torch.int32)
@@ -211,7 +213,7 @@ def make_config(index: int, *, seed: int = 0, layout: str = HEAD_MAJOR, num_seqs
 def make_test_shaped(*, batch_size: int, nheads: int, nheads_k: int, d: int, seqlen_k: int,
                      varlen: bool, has_sinks: bool, fp8: bool = False, block_size: int = 64,
                      seed: int = 0, dtype=torch.float16, layout: str = TOKEN_MAJOR,
-                     device="cpu") -> Workload:
+                     device="cpu", fp8_dtype=torch.float8_e5m2) -> Workload:
     """Inputs shaped like one case of the upstream test grid."""
     gen = torch.Generator(device="cpu")
     gen.manual_seed(seed)
@@ -228,8 +230,8 @@ def make_test_shaped(*, batch_size: int, nheads: int, nheads_k: int, d: int, seq
     else:
         lens = torch.full((batch_size,), seqlen_k, dtype=torch.int32)
     if fp8:
-        k = k.to(torch.float8_e5m2)
-        v = v.to(torch.float8_e5m2)
+        k = k.to(fp8_dtype)
+        v = v.to(fp8_dtype)
     sinks = torch.full((nheads,), 10.0, dtype=dtype) if has_sinks else None
     # upstream partition size: (head_size / 16) sub-groups x block_size tokens
     partition_size = (d // 16) * block_size if block_size == 64 else 512

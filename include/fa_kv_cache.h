@@ -23,6 +23,8 @@
  *                     FA_KV_CACHE_E5M2 : bytes, round-to-nearest-even of x / fp8_scale
  *                       (values beyond the E5M2 range become infinity, NaN stays NaN --
  *                       the behaviour of the tensor cast upstream uses)
+ *                     FA_KV_CACHE_E4M3 : the same with the 1-4-3 format, whose cast turns
+ *                       what lies beyond its range into NaN
  *   slot_mapping    [num_tokens] int64; token n goes to block slot / block_size, row
  *                   slot % block_size.  A negative slot, or one at or beyond
  *                   num_pool_blocks * block_size, is skipped (padding tokens).
@@ -39,7 +41,11 @@
 extern "C" {
 #endif
 
-typedef enum fa_kv_cache_dtype { FA_KV_CACHE_16BIT = 0, FA_KV_CACHE_E5M2 = 1 } fa_kv_cache_dtype;
+typedef enum fa_kv_cache_dtype {
+  FA_KV_CACHE_16BIT = 0,
+  FA_KV_CACHE_E5M2 = 1,
+  FA_KV_CACHE_E4M3 = 2 /* "fn" variant; beyond 448 becomes NaN, as torch.float8_e4m3fn casts */
+} fa_kv_cache_dtype;
 
 typedef struct fa_kv_cache_write_shape {
   int32_t num_tokens;

@@ -72,6 +72,12 @@ typedef enum fa_status {
 
 typedef enum fa_dtype { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 } fa_dtype;
 
+/* Byte format of an FP8 cache.  Upstream's FP8 kernels carry the format as a template
+ * parameter (paged_attention_kernel_fp8_loop.hpp:42) and its entry points fix E5M2
+ * (paged_attention_fp8_loop.cpp:43); E4M3 is the "fn" variant: bias 7, largest number 448,
+ * no infinities, 0x7f / 0xff NaN. */
+typedef enum fa_fp8_format { FA_FP8_E5M2 = 0, FA_FP8_E4M3 = 1 } fa_fp8_format;
+
 /* Shapes and strides that upstream reads off the torch tensors
  * (paged_attention_loop.cpp:60-65) or fixes at compile time. */
 typedef struct fa_paged_attention_shape {
@@ -108,7 +114,7 @@ typedef struct fa_paged_attention_options {
                                  upstream `run` returns (launch_kernels_loop.h:53,
                                  launch_kernels_reduce.h:76-77).  NULL: asynchronous, no timing. */
   int32_t validate_only;      /* non-zero: check arguments, launch nothing */
-  int32_t reserved;
+  int32_t kv_fp8_format;      /* FP8 entries only: fa_fp8_format of the caches; 0 = E5M2 as upstream */
 } fa_paged_attention_options;
 
 /* Single-pass kernel: one launch, no scratch. */

@@ -11,9 +11,9 @@
  * goes to slot_mapping[n] = block * block_size + row.
  *
  * Pinning status:
- *   oracle_f32_to_e5m2      pinned against the torch cast on every fp16 and every bf16
- *                           bit pattern and on fp32 values around every rounding boundary
- *                           (tests/test_oracle_kv_cache.py).
+ *   oracle_f32_to_e5m2,     pinned against the torch casts (float8_e5m2, float8_e4m3fn) on
+ *   oracle_f32_to_e4m3      every fp16 and every bf16 bit pattern and on fp32 values around
+ *                           every rounding boundary (tests/test_oracle_kv_cache.py).
  *   oracle_kv_cache_write   pinned against a torch index_put of cast tensors, both layouts,
  *                           skipped slots included.
  *   fp8_scale != 1          PARITY UNPINNED: upstream never quantises with a scale; the
@@ -68,6 +68,43 @@ ORACLE_API uint8_t oracle_f32_to_e5m2(float f) {
   return (uint8_t)(sign | out);
 }
 
+/* fp32 -> E4M3 "fn" (bias 7, 3 mantissa bits, no infinities), round to nearest, ties to
+ * even; what rounds beyond the largest number 448 (that is, 480 and above) becomes NaN, as
+ * the tensor cast to torch.float8_e4m3fn does; NaN is 0x7f with the sign kept. */
+ORACLE_API uint8_t oracle_f32_to_e4m3(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint8_t sign = (uint8_t)((x >> 24) & 0x80u);
+  uint32_t ax = x & 0x7FFFFFFFu;
+  if (ax >= 0x43F00000u) return (uint8_t)(sign | 0x7Fu); /* 480 and beyond, infinity, NaN */
+  if ((ax >> 23) == 0) return sign;                      /* zero and fp32 subnormals */
+  int32_t e = (int32_t)(ax >> 23) - 127;
+  uint64_t m = (ax & 0x7FFFFFu) | 0x800000u;
+  int32_t step_exp = e >= -6 ? e - 3 : -9; /* 3 mantissa bits; subnormal step 2^-9 */
+  int32_t shift = step_exp - (e - 23);
+  if (shift > 40) return sign;
+  uint64_t q = m >> shift;
+  uint64_t rem = m & (((uint64_t)1 << shift) - 1);
+  uint64_t half = (uint64_t)1 << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) q++;
+  uint32_t out;
+  if (e >= -6) {
+    uint32_t be = (uint32_t)(e + 7);
+    if (q == 16) {
+      be += 1;
+      q = 8;
+    }
+    out = (be << 3) | (uint32_t)(q - 8);
+  } else {
+    out = (uint32_t)q; /* 0..8; 8 is the smallest normal */
+  }
+  return (uint8_t)(sign | out);
+}
+
+ORACLE_API void oracle_f32_to_e4m3_array(const float *src, uint8_t *dst, int64_t n) {
+  for (int64_t k = 0; k < n; ++k) dst[k] = oracle_f32_to_e4m3(src[k]);
+}
+
 ORACLE_API void oracle_f32_to_e5m2_array(const float *src, uint8_t *dst, int64_t n) {
   for (int64_t k = 0; k < n; ++k) dst[k] = oracle_f32_to_e5m2(src[k]);
 }
@@ -77,7 +114,7 @@ typedef struct oracle_kv_write {
   int64_t kv_block_stride, kv_token_stride, kv_head_stride; /* elements */
   int64_t src_token_stride, src_head_stride;                /* elements */
   int32_t src_dtype;   /* 0 fp16, 1 bf16 */
-  int32_t cache_dtype; /* 0 16-bit copy, 1 E5M2 */
+  int32_t cache_dtype; /* 0 16-bit copy, 1 E5M2, 2 E4M3 */
   int64_t num_pool_blocks;
   float fp8_scale;
 } oracle_kv_write;
@@ -90,7 +127,7 @@ static void write_row(const uint16_t *src, void *cache, int64_t dst, const oracl
   uint8_t *out = (uint8_t *)cache + dst;
   for (int d = 0; d < w->head_size; ++d) {
     float x = w->src_dtype == 1 ? oracle_bf16_to_f32(src[d]) : oracle_f16_to_f32(src[d]);
-    out[d] = oracle_f32_to_e5m2(x * inv);
+    out[d] = w->cache_dtype == 2 ? oracle_f32_to_e4m3(x * inv) : oracle_f32_to_e5m2(x * inv);
   }
 }
 

@@ -20,7 +20,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle_paged_attention.so")
 _lib = None
 
 Q_F16, Q_BF16 = 0, 1
-KV_SAME_AS_Q, KV_E5M2 = 0, 1
+KV_SAME_AS_Q, KV_E5M2, KV_E4M3 = 0, 1, 2
 
 
 class _Problem(ctypes.Structure):
@@ -95,6 +95,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_num_threads.restype = ctypes.c_int
         L.oracle_f32_to_e5m2.argtypes = [ctypes.c_float]
         L.oracle_f32_to_e5m2.restype = ctypes.c_uint8
+        L.oracle_f32_to_e4m3_array.argtypes = [P, P, ctypes.c_int64]
+        L.oracle_f32_to_e4m3_array.restype = None
+        L.oracle_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+        L.oracle_e4m3_to_f32.restype = ctypes.c_float
         L.oracle_f32_to_e5m2_array.argtypes = [P, P, ctypes.c_int64]
         L.oracle_f32_to_e5m2_array.restype = None
         L.oracle_kv_cache_write.argtypes = [P, P, P, P, P, ctypes.POINTER(_KvWrite)]
@@ -118,7 +122,7 @@ def _problem(query, key_cache, value_cache, block_tables, context_lens, scale, b
              kv_strides, fp8_scale, num_kv_heads):
     assert query.device.type == "cpu" and query.is_contiguous() and query.dim() == 3
     assert query.dtype in (torch.float16, torch.bfloat16)
-    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.uint8)
+    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8)
     if not fp8:
         assert key_cache.dtype == query.dtype, "16-bit caches share the query dtype"
     assert value_cache.dtype == key_cache.dtype
@@ -131,7 +135,7 @@ def _problem(query, key_cache, value_cache, block_tables, context_lens, scale, b
     pr.max_blocks_per_seq = block_tables.shape[1]
     pr.kv_block_stride, pr.kv_token_stride, pr.kv_head_stride = kv_strides
     pr.q_dtype = Q_BF16 if query.dtype == torch.bfloat16 else Q_F16
-    pr.kv_dtype = KV_E5M2 if fp8 else KV_SAME_AS_Q
+    pr.kv_dtype = (KV_E4M3 if key_cache.dtype == torch.float8_e4m3fn else KV_E5M2) if fp8 else KV_SAME_AS_Q
     pr.scale = scale
     pr.fp8_scale = fp8_scale
     return pr
@@ -212,6 +216,14 @@ def kernel_reduce(exp_sums, max_logits, tmp_out, context_lens, *, partition_size
     return (out, out32) if want_f32 else out
 
 
+def f32_to_e4m3(values: torch.Tensor) -> torch.Tensor:
+    """Element-wise fp32 -> E4M3 "fn" byte (round to nearest even, beyond 448 to NaN)."""
+    src = values.to(torch.float32).contiguous()
+    out = torch.empty(src.shape, dtype=torch.uint8)
+    lib().oracle_f32_to_e4m3_array(_ptr(src), _ptr(out), ctypes.c_int64(src.numel()))
+    return out
+
+
 def f32_to_e5m2(values: torch.Tensor) -> torch.Tensor:
     """Element-wise fp32 -> E5M2 byte (round to nearest even, overflow to infinity)."""
     src = values.to(torch.float32).contiguous()
@@ -221,14 +233,14 @@ def f32_to_e5m2(values: torch.Tensor) -> torch.Tensor:
 
 
 def kv_cache_write(key, value, key_cache, value_cache, slot_mapping, *, block_size, kv_strides,
-                   fp8_scale=1.0):
+                   fp8_scale=1.0, e4m3=False):
     """Scatter the rows of `key`/`value` ([N, Hk, D], fp16/bf16) into the paged pools in place
     (the pool build of test_paged_fp8cache.py:171-203 as a per-token scatter)."""
     assert key.device.type == "cpu" and key.dim() == 3 and key.stride(2) == 1
     assert value.shape == key.shape and value.stride() == key.stride() and value.dtype == key.dtype
     assert key.dtype in (torch.float16, torch.bfloat16)
     assert slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous()
-    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.uint8)
+    fp8 = key_cache.dtype in (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8) or e4m3
     if not fp8:
         assert key_cache.dtype == key.dtype
     assert value_cache.dtype == key_cache.dtype and key_cache.is_contiguous() and value_cache.is_contiguous()
@@ -238,7 +250,7 @@ def kv_cache_write(key, value, key_cache, value_cache, slot_mapping, *, block_si
     w.kv_block_stride, w.kv_token_stride, w.kv_head_stride = kv_strides
     w.src_token_stride, w.src_head_stride = key.stride(0), key.stride(1)
     w.src_dtype = Q_BF16 if key.dtype == torch.bfloat16 else Q_F16
-    w.cache_dtype = KV_E5M2 if fp8 else KV_SAME_AS_Q
+    w.cache_dtype = (KV_E4M3 if (e4m3 or key_cache.dtype == torch.float8_e4m3fn) else KV_E5M2) if fp8 else KV_SAME_AS_Q
     w.num_pool_blocks = key_cache.shape[0]
     w.fp8_scale = fp8_scale
     lib().oracle_kv_cache_write(_ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache),

@@ -35,7 +35,8 @@
  *                            float64 brute force, closed forms and invariants.
  *   oracle_kernel_*          pinned against oracle_attention_ref through the
  *                            split-invariance of log-sum-exp and by closed forms.
- *   e5m2 decode              pinned on all 256 codes against torch.float8_e5m2.
+ *   e5m2 / e4m3 decode       pinned on all 256 codes against torch.float8_e5m2 /
+ *                            torch.float8_e4m3fn.
  *   fp8_scale != 1           PARITY UNPINNED: the upstream tests only ever pass
  *                            1.0 (test_paged_fp8cache.py:489,510); the reading
  *                            implemented is K^ = dequant(K)*s, V^ = dequant(V)*s.
@@ -56,7 +57,7 @@
 #define CLONES __attribute__((target_clones("avx2", "default")))
 
 enum { ORACLE_Q_F16 = 0, ORACLE_Q_BF16 = 1 };
-enum { ORACLE_KV_SAME_AS_Q = 0, ORACLE_KV_E5M2 = 1 };
+enum { ORACLE_KV_SAME_AS_Q = 0, ORACLE_KV_E5M2 = 1, ORACLE_KV_E4M3 = 2 };
 
 /* ------------------------------------------------------------------ */
 /* 16-bit and 8-bit float formats, bit exact, round-to-nearest-even     */
@@ -133,6 +134,19 @@ ORACLE_API uint16_t oracle_f32_to_bf16(float f) {
 /* E5M2 is binary16 cut down to its top byte, so decoding is a byte shift. */
 ORACLE_API float oracle_e5m2_to_f32(uint8_t b) { return oracle_f16_to_f32((uint16_t)((uint16_t)b << 8)); }
 
+/* E4M3 ("fn": finite numbers and NaN only): 1 sign, 4 exponent bits with bias 7, 3 mantissa
+ * bits; exponent 15 with mantissa 7 is NaN, everything else is a number (largest 448);
+ * exponent 0 holds the subnormals m * 2^-9.  The format upstream's FP8 kernels carry as a
+ * template parameter next to E5M2 (paged_attention_kernel_fp8_loop.hpp:42). */
+ORACLE_API float oracle_e4m3_to_f32(uint8_t b) {
+  const int sign = b >> 7, e = (b >> 3) & 15, m = b & 7;
+  float v;
+  if (e == 15 && m == 7) return bits_to_f32(sign ? 0xFFC00000u : 0x7FC00000u);
+  if (e == 0) v = (float)m * 0.001953125f; /* m * 2^-9 */
+  else v = ldexpf((float)(8 + m), e - 10); /* (1 + m/8) * 2^(e-7) */
+  return sign ? -v : v;
+}
+
 static inline float load16(const uint16_t *p, int q_dtype) {
   return q_dtype == ORACLE_Q_BF16 ? oracle_bf16_to_f32(*p) : oracle_f16_to_f32(*p);
 }
@@ -172,6 +186,9 @@ CLONES static void gather_rows(float *dst, const void *cache, const int32_t *tab
     if (p->kv_dtype == ORACLE_KV_E5M2) {
       const uint8_t *src = (const uint8_t *)cache + off;
       for (int d = 0; d < D; ++d) row[d] = oracle_e5m2_to_f32(src[d]) * p->fp8_scale;
+    } else if (p->kv_dtype == ORACLE_KV_E4M3) {
+      const uint8_t *src = (const uint8_t *)cache + off;
+      for (int d = 0; d < D; ++d) row[d] = oracle_e4m3_to_f32(src[d]) * p->fp8_scale;
     } else {
       const uint16_t *src = (const uint16_t *)cache + off;
       if (p->q_dtype == ORACLE_Q_BF16)
@@ -300,8 +317,8 @@ ORACLE_API int oracle_kernel_loop(uint16_t *out, float *out_f32, const uint16_t 
   const int G = H / Hk;
   oracle_problem raw = *p;
   raw.fp8_scale = 1.0f; /* rows without the scale; folded in after the dots */
-  const float kscale = p->kv_dtype == ORACLE_KV_E5M2 ? p->scale * p->fp8_scale : p->scale;
-  const float vscale = p->kv_dtype == ORACLE_KV_E5M2 ? p->fp8_scale : 1.0f;
+  const float kscale = p->kv_dtype != ORACLE_KV_SAME_AS_Q ? p->scale * p->fp8_scale : p->scale;
+  const float vscale = p->kv_dtype != ORACLE_KV_SAME_AS_Q ? p->fp8_scale : 1.0f;
   int failed = 0;
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
   for (int s = 0; s < S; ++s) {
@@ -386,8 +403,8 @@ ORACLE_API int oracle_kernel_partition(float *exp_sums, float *max_logits, float
   const int G = H / Hk;
   oracle_problem raw = *p;
   raw.fp8_scale = 1.0f;
-  const float kscale = p->kv_dtype == ORACLE_KV_E5M2 ? p->scale * p->fp8_scale : p->scale;
-  const float vscale = p->kv_dtype == ORACLE_KV_E5M2 ? p->fp8_scale : 1.0f;
+  const float kscale = p->kv_dtype != ORACLE_KV_SAME_AS_Q ? p->scale * p->fp8_scale : p->scale;
+  const float vscale = p->kv_dtype != ORACLE_KV_SAME_AS_Q ? p->fp8_scale : 1.0f;
   int failed = 0;
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
   for (int s = 0; s < S; ++s) {

@@ -18,7 +18,7 @@ def dense_kv(w, cache):
     B = w.block_size
     max_ctx = int(w.context_lens.max())
     nb = (max_ctx + B - 1) // B
-    c = cache.to(w.query.dtype).float() if cache.dtype == torch.float8_e5m2 else cache.float()
+    c = cache.to(w.query.dtype).float() if cache.dtype in (torch.float8_e5m2, torch.float8_e4m3fn) else cache.float()
     if w.layout == "head_major":
         c = c.permute(0, 2, 1, 3)  # -> [NB, B, Hk, D]
     idx = w.block_tables[:, :nb].long()
@@ -57,7 +57,7 @@ def brute_force(w):
     def row(cache, s, t, kh):
         blk = int(w.block_tables[s, t // B])
         r = cache[blk, kh, t % B] if w.layout == "head_major" else cache[blk, t % B, kh]
-        if r.dtype == torch.float8_e5m2:
+        if r.dtype in (torch.float8_e5m2, torch.float8_e4m3fn):
             r = r.to(w.query.dtype)
         return r.double() * w.fp8_scale
 

@@ -54,9 +54,10 @@ def _shape(**kw):
     return s
 
 
-def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0):
+def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0):
     op = _cabi.Options()
     op.validate_only = 1
+    op.kv_fp8_format = fp8_format
     name = "fa_paged_attention_" + ("fp8_" if fp8 else "") + ("reduce" if split else "loop")
     args = [ptr, ptr, ptr, ptr, ptr, ptr, 0.1, max_ctx]
     if split:
@@ -70,6 +71,13 @@ def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max
 def test_valid_arguments_pass(L, split, fp8):
     rc, msg = _call(L, split, fp8)
     assert rc == _cabi.FA_OK and msg == ""
+
+
+def test_fp8_format_is_checked_on_fp8_entries_only(L):
+    assert _call(L, fp8=True, fp8_format=_cabi.FA_FP8_E4M3)[0] == _cabi.FA_OK
+    assert _call(L, fp8=True, split=True, fp8_format=_cabi.FA_FP8_E4M3)[0] == _cabi.FA_OK
+    assert _call(L, fp8=True, fp8_format=7)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
+    assert _call(L, fp8=False, fp8_format=7)[0] == _cabi.FA_OK   # 16-bit entries ignore the field
 
 
 def test_error_codes(L):
@@ -146,7 +154,8 @@ def test_kv_cache_write_argument_checks(L):
     assert _kv_write(L, ptr=0)[0] == _cabi.FA_ERR_NULL_POINTER
     assert _kv_write(L, slots=0)[0] == _cabi.FA_ERR_NULL_POINTER
     assert _kv_write(L, src_dtype=5)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
-    assert _kv_write(L, cache_dtype=2)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
+    assert _kv_write(L, cache_dtype=_cabi.FA_KV_CACHE_E4M3)[0] == _cabi.FA_OK
+    assert _kv_write(L, cache_dtype=3)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
     assert _kv_write(L, head_size=100)[0] == _cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE
     assert _kv_write(L, num_pool_blocks=0)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _kv_write(L, kv_token_stride=64)[0] == _cabi.FA_ERR_BAD_SHAPE       # shorter than a row

@@ -60,6 +60,24 @@ def test_every_16bit_pattern(oracle, src, scale):
         assert torch.equal(wk.view(-1), x.to(torch.float8_e5m2).view(torch.uint8).view(-1))
 
 
+@pytest.mark.parametrize("src", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("scale", [1.0, 0.5, 3.0])
+def test_every_16bit_pattern_e4m3(oracle, src, scale):
+    dev = _dev()
+    x = _all_16bit(src).view(512, 1, 128)
+    y = x.flip(0).contiguous()
+    slots = torch.arange(512, dtype=torch.int64)
+    wk, wv = torch.zeros((512, 1, 1, 128), dtype=torch.uint8), torch.zeros((512, 1, 1, 128), dtype=torch.uint8)
+    oracle.kv_cache_write(x, y, wk, wv, slots, block_size=1, kv_strides=(128, 128, 128), fp8_scale=scale, e4m3=True)
+    gk = torch.zeros((512, 1, 1, 128), dtype=torch.float8_e4m3fn, device=dev)
+    gv = torch.zeros_like(gk)
+    kv_cache_write.run(x.to(dev), y.to(dev), gk, gv, slots.to(dev), scale)
+    torch.cuda.synchronize()
+    assert torch.equal(gk.view(torch.uint8).cpu(), wk) and torch.equal(gv.view(torch.uint8).cpu(), wv)
+    if scale == 1.0:  # and the oracle's bytes are torch's
+        assert torch.equal(wk.view(-1), x.to(torch.float8_e4m3fn).view(torch.uint8).view(-1))
+
+
 @pytest.mark.parametrize("layout", [W.TOKEN_MAJOR, W.HEAD_MAJOR])
 @pytest.mark.parametrize("src", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("fp8", [False, True])

@@ -301,6 +301,48 @@ def test_table_wider_than_the_persistent_loop_key(oracle):
     _check(bufs.out, w, oracle, "2^24-token table/loop")
 
 
+@pytest.mark.parametrize("qdtype", [torch.float16, torch.bfloat16])
+def test_e4m3_caches(oracle, qdtype):
+    """FP8 caches in the E4M3 format (torch.float8_e4m3fn pools) through all four FP8 code
+    paths: loop and split kernels, head sizes 128 and 64, with sinks and a non-unit scale."""
+    cases = [
+        W.make_test_shaped(batch_size=3, nheads=8, nheads_k=2, d=128, seqlen_k=1500, varlen=True, has_sinks=True,
+                           fp8=True, dtype=qdtype, fp8_dtype=torch.float8_e4m3fn),
+        W.make_test_shaped(batch_size=2, nheads=6, nheads_k=6, d=64, seqlen_k=333, varlen=True, has_sinks=False,
+                           fp8=True, dtype=qdtype, fp8_dtype=torch.float8_e4m3fn, block_size=16, layout=W.HEAD_MAJOR),
+    ]
+    cases[1].fp8_scale = 0.5
+    if qdtype == torch.float16:
+        cases.append(W.make_config(3, num_seqs=6, pool_blocks=800, fp8_dtype=torch.float8_e4m3fn))
+    else:
+        cases.append(W.make_config(4, num_seqs=5, pool_blocks=8192, fp8_dtype=torch.float8_e4m3fn))
+    for w in cases:
+        assert w.key_cache.dtype == torch.float8_e4m3fn
+        for kernel in ("fp8_loop", "fp8_reduce"):
+            bufs, _ = _run(w, kernel)
+            _check(bufs.out, w, oracle, f"e4m3 {w.name}/{kernel}")
+
+
+def test_e4m3_special_bytes(oracle):
+    """Every E4M3 byte as a K and a V value (NaN codes kept beyond the context): the decode
+    agrees with the oracle's table on all 254 numbers, subnormals included."""
+    w = W.make_test_shaped(batch_size=1, nheads=2, nheads_k=1, d=64, seqlen_k=256, varlen=False, has_sinks=False,
+                           fp8=True, fp8_dtype=torch.float8_e4m3fn, block_size=64)
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    numbers = codes[(codes & 0x7f) != 0x7f]                       # all but the two NaN codes
+    vals = numbers[torch.randperm(254, generator=torch.Generator().manual_seed(0))]
+    kc = w.key_cache.view(torch.uint8).view(-1)
+    vc = w.value_cache.view(torch.uint8).view(-1)
+    kc.copy_(vals.repeat(kc.numel() // 254 + 1)[:kc.numel()])
+    vc.copy_(vals.flip(0).repeat(vc.numel() // 254 + 1)[:vc.numel()])
+    w.scale = 1e-4                                                 # keeps the logits of +-448 values finite
+    bufs, _ = _run(w, "fp8_loop")
+    ref = call_oracle(oracle.attention_ref, w, want_f32=True)[1]
+    got = bufs.out.float().cpu()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, ref, atol=5e-2, rtol=1e-2)    # values up to 448: the bar scales with them
+
+
 def test_bf16_and_fp8_scale(oracle):
     # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
     w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,

@@ -24,6 +24,8 @@ def _grid_case(**kw):
     dict(fp8=True, nheads=14, nheads_k=2, seqlen_k=799, has_sinks=True),
     dict(layout=W.HEAD_MAJOR, block_size=16, seqlen_k=257),
     dict(dtype=torch.bfloat16, fp8=True, d=128, seqlen_k=1024, has_sinks=True),
+    dict(fp8=True, fp8_dtype=torch.float8_e4m3fn, nheads=6, nheads_k=2, seqlen_k=500, has_sinks=True),
+    dict(dtype=torch.bfloat16, fp8=True, fp8_dtype=torch.float8_e4m3fn, d=128, seqlen_k=300),
 ])
 def test_attention_ref_equals_sdpa(oracle, kw):
     w = _grid_case(**kw)

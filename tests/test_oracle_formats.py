@@ -42,6 +42,17 @@ def test_e5m2_decode_all_256_codes(oracle):
     assert np.isnan(got[~ok.numpy()]).all()
 
 
+def test_e4m3_decode_all_256_codes(oracle):
+    """E4M3 "fn" decode against torch.float8_e4m3fn, NaN codes included."""
+    L = oracle.lib()
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    want = codes.view(torch.float8_e4m3fn).float().numpy()
+    got = _vec(lambda c: L.oracle_e4m3_to_f32(int(c)), codes.numpy(), np.float32)
+    ok = ~np.isnan(want)
+    assert np.array_equal(got.view(np.uint32)[ok], want.view(np.uint32)[ok])
+    assert np.isnan(got[~ok]).all() and (~ok).sum() == 2
+
+
 def _encode_cases():
     rng = np.random.default_rng(0)
     xs = [rng.standard_normal(20000).astype(np.float32),

@@ -42,6 +42,49 @@ def test_cast_matches_torch_around_every_rounding_boundary(oracle):
     assert torch.equal(oracle.f32_to_e5m2(r), r.to(torch.float8_e5m2).view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_e4m3_cast_matches_torch_on_every_16bit_pattern(oracle, dtype):
+    x = _all_16bit(dtype)
+    assert torch.equal(oracle.f32_to_e4m3(x.float()), x.to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+def test_e4m3_cast_matches_torch_around_every_rounding_boundary(oracle):
+    codes = torch.arange(0, 0x7f, dtype=torch.uint8)            # non-negative numbers, 448 the largest
+    vals = codes.view(torch.float8_e4m3fn).float().double().numpy()
+    pts = []
+    for a, b in zip(vals[:-1], vals[1:]):
+        mid = np.float32((a + b) / 2)
+        pts += [np.float32(a), mid, np.nextafter(mid, np.float32(np.inf), dtype=np.float32),
+                np.nextafter(mid, np.float32(-np.inf), dtype=np.float32)]
+    pts += [np.float32(448.0), np.float32(464.0), np.nextafter(np.float32(464.0), np.float32(0), dtype=np.float32),
+            np.nextafter(np.float32(464.0), np.float32(np.inf), dtype=np.float32), np.float32(479.99),
+            np.nextafter(np.float32(480.0), np.float32(0), dtype=np.float32), np.float32(480.0), np.float32(512.0),
+            np.float32(1e30), np.float32(np.inf), np.float32(2.0 ** -10),
+            np.nextafter(np.float32(2.0 ** -10), np.float32(1), dtype=np.float32), np.float32(2.0 ** -11),
+            np.float32(1e-30), np.float32(1e-45), np.float32(0.0)]
+    x = torch.from_numpy(np.array(pts, dtype=np.float32))
+    x = torch.cat([x, -x])
+    assert torch.equal(oracle.f32_to_e4m3(x), x.to(torch.float8_e4m3fn).view(torch.uint8))
+    g = torch.Generator().manual_seed(0)
+    r = torch.randn(200000, generator=g) * torch.exp(torch.randn(200000, generator=g) * 4)
+    assert torch.equal(oracle.f32_to_e4m3(r), r.to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+def test_e4m3_writer_matches_torch_indexing(oracle):
+    g = torch.Generator().manual_seed(4)
+    N, Hk, D, B, NB = 29, 2, 64, 16, 4
+    key = (torch.randn(N, Hk, D, generator=g) * 100).to(torch.float16)    # some beyond 448
+    value = (torch.randn(N, Hk, D, generator=g) * 2).to(torch.float16)
+    slots = torch.randperm(NB * B, generator=g)[:N].to(torch.int64)
+    kc = torch.full((NB, B, Hk, D), 9, dtype=torch.uint8)
+    vc = torch.full((NB, B, Hk, D), 9, dtype=torch.uint8)
+    want_k, want_v = kc.clone(), vc.clone()
+    want_k.view(NB * B, Hk, D)[slots] = key.to(torch.float8_e4m3fn).view(torch.uint8)
+    want_v.view(NB * B, Hk, D)[slots] = value.to(torch.float8_e4m3fn).view(torch.uint8)
+    oracle.kv_cache_write(key, value, kc, vc, slots, block_size=B, kv_strides=(B * Hk * D, Hk * D, D), e4m3=True)
+    assert torch.equal(kc, want_k) and torch.equal(vc, want_v)
+
+
 def _pool(layout, NB, B, Hk, D, dtype, fill):
     shape = (NB, B, Hk, D) if layout == "token_major" else (NB, Hk, B, D)
     if dtype == torch.float8_e5m2:
