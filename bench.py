@@ -51,8 +51,8 @@ def _clones(w, torch):
     return ks, vs
 
 
-def _build_config(index, torch, W, runner, dev):
-    w = W.make_config(index, device=dev, pools_on_device=True)
+def _build_config(index, torch, W, runner, dev, **kw):
+    w = W.make_config(index, device=dev, pools_on_device=True, **kw)
     ks, vs = _clones(w, torch)
     return w, ks, vs
 
@@ -276,6 +276,12 @@ def main():
                      "kernel_us": kernel_us},
         "configs": others,
     }
+    # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
+    e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
+    _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+    r["workload"] += "_e4m3"
+    others.append(r)
+    del e4m3
     line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
         del built
