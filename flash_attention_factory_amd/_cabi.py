@@ -40,6 +40,10 @@ FA_KV_CACHE_E4M3 = 2
 FA_FP8_E5M2 = 0
 FA_FP8_E4M3 = 1
 
+FA_MASK_ALIBI = 1
+FA_MASK_SOFTCAP = 2
+FA_MASK_WINDOW = 4
+
 
 class Shape(ctypes.Structure):
     _fields_ = [
@@ -69,6 +73,8 @@ class Options(ctypes.Structure):
         ("elapsed_us", ctypes.POINTER(ctypes.c_float)),
         ("validate_only", ctypes.c_int32),
         ("kv_fp8_format", ctypes.c_int32),
+        ("mask_flags", ctypes.c_int32),
+        ("window_left", ctypes.c_int32),
     ]
 
 

@@ -55,6 +55,10 @@ struct Resolved {
   int32_t kv_elem_bytes;
   float fp8_scale;
   bool e4m3;  // FP8 entries: the caches hold E4M3 bytes, not E5M2
+  int32_t mask_flags;  // fa_mask bits to apply
+  const float *alibi_slopes;
+  float softcap;
+  int32_t window_left;
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -125,6 +129,18 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   if (kv8 && o && o->kv_fp8_format != FA_FP8_E5M2 && o->kv_fp8_format != FA_FP8_E4M3)
     return fail(FA_ERR_UNSUPPORTED_DTYPE, "kv_fp8_format %d is neither E5M2 (0) nor E4M3 (1)", o->kv_fp8_format);
   r->e4m3 = kv8 && o && o->kv_fp8_format == FA_FP8_E4M3;
+  r->mask_flags = o ? o->mask_flags : 0;
+  if (r->mask_flags & ~(FA_MASK_ALIBI | FA_MASK_SOFTCAP | FA_MASK_WINDOW))
+    return fail(FA_ERR_BAD_SHAPE, "mask_flags 0x%x has bits that mean nothing", r->mask_flags);
+  if ((r->mask_flags & FA_MASK_ALIBI) && !o->alibi_slopes)
+    return fail(FA_ERR_NULL_POINTER, "FA_MASK_ALIBI needs alibi_slopes");
+  if ((r->mask_flags & FA_MASK_SOFTCAP) && !(o->softcap > 0.f))
+    return fail(FA_ERR_BAD_SHAPE, "FA_MASK_SOFTCAP needs softcap > 0");
+  if ((r->mask_flags & FA_MASK_WINDOW) && o->window_left < 0)
+    return fail(FA_ERR_BAD_SHAPE, "FA_MASK_WINDOW needs window_left >= 0");
+  r->alibi_slopes = o ? o->alibi_slopes : nullptr;
+  r->softcap = o ? o->softcap : 0.f;
+  r->window_left = o ? o->window_left : 0;
   r->fp8_scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
   r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   r->elapsed_us = o ? o->elapsed_us : nullptr;
@@ -148,6 +164,11 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.context_lens = context_lens;
   p.sinks = r.sinks;
   p.score_scale_log2 = scale * r.fp8_scale * kLog2e;
+  p.score_scale = scale * r.fp8_scale;
+  p.mask_flags = r.mask_flags;
+  p.alibi_slopes = r.alibi_slopes;
+  p.softcap = r.softcap;
+  p.window_left = r.window_left;
   p.out_scale = r.fp8_scale;
   p.num_seqs = s.num_seqs;
   p.num_heads = s.num_heads;

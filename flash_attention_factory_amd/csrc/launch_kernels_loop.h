@@ -28,8 +28,15 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
   const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
-  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
-      max_ctx < kLoopPersistentMaxContext) {
+  if (r.mask_flags != 0) {
+    // score modifiers: the grid form has the instance that applies them
+    const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+    FA_HIP_CHECK(timer.launch(
+        paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
+                          Pipeline<KV8>::tiles_per_chunk, true>,
+        grid, dim3(NW * 64), 0, p));
+  } else if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
+             max_ctx < kLoopPersistentMaxContext) {
     // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
     // sequences first, with the next item's first loads issued before each merge.
     constexpr int PW = PersistentLoop<KV8>::waves;

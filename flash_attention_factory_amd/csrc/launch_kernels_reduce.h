@@ -32,7 +32,14 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // work-group per (kv head, partition slot, sequence); slots past a sequence's length
   // return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
   int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
-  if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
+  if (r.mask_flags != 0) {
+    // score modifiers: the grid form has the instance that applies them
+    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+    FA_HIP_CHECK(timer.launch(
+        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
+                          Pipeline<KV8>::tiles_per_chunk, true>,
+        grid, dim3(NW * 64), 0, p));
+  } else if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
       (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
     // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
     constexpr int SW = SegmentSplit<KV8>::waves;

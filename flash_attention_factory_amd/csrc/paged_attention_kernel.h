@@ -72,7 +72,7 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   }
 
   if (i >= p.group) return;
-  const float inv = p.out_scale / L;
+  const float inv = L > 0.f ? p.out_scale / L : 0.f;  // L = 0: a partition wholly before a local window
   const int head = kvh * p.group + i;
   const int d0 = 4 * r * NDT + wave * SL;  // first head-dim element this lane stores
   if constexpr (PART) {
@@ -89,7 +89,10 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   }
 }
 
-template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC>
+// MASKS: an instance that also applies the score modifiers of p.mask_flags (soft-capping,
+// local window, ALiBi).  Chunks that lie wholly before a sequence's window are skipped; a
+// partition that lies wholly before it stores an empty partial (max -inf, sum 0, zeros).
+template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC, bool MASKS = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {
   using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop>;
@@ -126,14 +129,19 @@ paged_attn_kernel(const PagedAttnParams p) {
 
   wa.load_q(seq, kvh);
   wa.reset(wa.load_sink(kvh, wave == 0 && (!PART || part == 0)));
+  int c_lo = c_begin;  // first chunk that holds a visible token
+  if constexpr (MASKS) {
+    wa.load_slope(kvh);
+    if (p.mask_flags & kMaskWindow) c_lo = max(c_begin, max(0, ctx - 1 - p.window_left) / CT);
+  }
 
   // ---- streaming loop ------------------------------------------------------------------
   // The last chunk of a wavefront is computed outside the issuing path, so no wait on the
   // loads of the current chunk ever has to cover a path on which nothing more was issued.
   // Only that last chunk can reach past the end of the token range.
-  int ci = c_begin + wave;
+  int ci = c_lo + wave;
   if (ci < c_end) {
-    if (!pool_known) ids0 = wa.fetch_ids(table, ci, last_blk);
+    if (!pool_known || c_lo != c_begin) ids0 = wa.fetch_ids(table, ci, last_blk);
     // One register set.  K of chunk n+1 is requested as soon as the score MFMAs of
     // chunk n have read K, V of chunk n+1 as soon as the P.V MFMAs have read V: about
     // half a chunk is in flight per wavefront at any time.  (Two register sets with the
@@ -147,14 +155,14 @@ paged_attn_kernel(const PagedAttnParams p) {
       const int cn = ci + NW;
       const auto s = wa.qk(R);
       wa.issue_k(R, kvh, cn, nids);
-      const auto pb = wa.template soft<false>(R, s, ci, tok_end);
+      const auto pb = wa.template soft<false, MASKS>(R, s, ci, tok_end, ctx - 1);
       wa.pv(R, pb);
       wa.issue_v(R, kvh, cn, nids);
       nids = wa.fetch_ids(table, cn + NW, last_blk);
       ci = cn;
     }
     const auto s = wa.qk(R);
-    wa.pv(R, wa.template soft<true>(R, s, ci, tok_end));
+    wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end, ctx - 1));
   }
 
   merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part);

@@ -48,7 +48,15 @@ struct PagedAttnParams {
   int64_t kv_block_bytes;       // strides in BYTES
   int64_t kv_token_bytes;
   int64_t kv_head_bytes;
+  // score modifiers, applied only by kernel instances built with MASKS (mask_flags != 0)
+  const float *alibi_slopes;    // [H] fp32
+  float score_scale;            // sm_scale * fp8_scale (natural-log units)
+  float softcap;
+  int32_t window_left;
+  int32_t mask_flags;           // kMaskAlibi | kMaskSoftcap | kMaskWindow
 };
+
+constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
 
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
@@ -90,9 +98,15 @@ struct WaveAttn {
   // acc[dt][e]: O^T[d = (4r+e)*NDT + dt][head i], un-normalised.
   float m, l;
   f32x4 acc[NDT];
+  float slope_log2 = 0.f;  // ALiBi slope of head i in base-2 units (MASKS instances only)
 
   __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
       : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {}
+
+  // ALiBi slope of this lane's head; kernels built with MASKS call it once per item.
+  __device__ __forceinline__ void load_slope(int kvh) {
+    slope_log2 = ((p.mask_flags & kMaskAlibi) && i < p.group) ? p.alibi_slopes[kvh * p.group + i] * kLog2e : 0.f;
+  }
 
   __device__ __forceinline__ void load_q(int seq, int kvh) {
     const int head = kvh * p.group + i;
@@ -222,12 +236,32 @@ struct WaveAttn {
   // Online softmax step over the chunk's tokens; returns the P^T "B" operands.
   // check_tail: whether this chunk can reach past tok_end (a compile-time false drops
   // the masking code from the steady-state loop).
-  template <bool CHECK_TAIL>
-  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end) {
+  // MASKS: apply the score modifiers p.mask_flags names -- soft-capping, local window, ALiBi,
+  // in that order (upstream test_paged.py:92-110) -- for a query at position `last_pos`.
+  // The caller never hands over a chunk that lies wholly before the window.
+  template <bool CHECK_TAIL, bool MASKS = false>
+  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end, int last_pos = 0) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
     float t[NT];
+    if constexpr (MASKS) {
+      const bool cap = p.mask_flags & kMaskSoftcap;
+      const float inv_cap2 = 2.0f * kLog2e / p.softcap;  // exp(2x/cap) = exp2(x * inv_cap2)
+      const int first_visible = (p.mask_flags & kMaskWindow) ? last_pos - p.window_left : 0;
 #pragma unroll
-    for (int e = 0; e < NT; ++e) t[e] = s.v[e >> 2][e & 3] * p.score_scale_log2;
+      for (int e = 0; e < NT; ++e) {
+        float x = s.v[e >> 2][e & 3] * p.score_scale;
+        if (cap) {  // cap * tanh(x / cap), tanh(z) = 1 - 2 / (exp(2z) + 1)
+          const float e2 = fast_exp2(x * inv_cap2);
+          x = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f));
+        }
+        const int tok = ci * CT + (e >> 2) * kTileTokens + 4 * r + (e & 3);
+        x = x * kLog2e + slope_log2 * (float)(tok - last_pos);
+        t[e] = tok < first_visible ? -INFINITY : x;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < NT; ++e) t[e] = s.v[e >> 2][e & 3] * p.score_scale_log2;
+    }
     if constexpr (CHECK_TAIL) {
       const int t0 = ci * CT;
       if (t0 + CT > tok_end) {  // wave-uniform

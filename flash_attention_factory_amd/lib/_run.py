@@ -39,7 +39,8 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
              debug_output, query, key_cache, value_cache, block_tables, context_lens,
              num_queries_per_tokens: int, sm_scale: float, fp8_scale: float, block_size: int,
              max_context_len: int, alibi_slopes, sinks: Optional[torch.Tensor], softcap: float,
-             partition_size: int = 0, timed: bool = True) -> List[float]:
+             partition_size: int = 0, timed: bool = True, apply_alibi: bool = False,
+             apply_softcap: bool = False, window_left: Optional[int] = None) -> List[float]:
     L = _cabi.load()
     if not query.is_cuda:
         raise RuntimeError("paged attention runs on the GPU only: `query` is not a device tensor")
@@ -85,6 +86,17 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     op.alibi_slopes = alibi_slopes.data_ptr() if alibi_slopes is not None else None
     op.softcap = softcap
     op.fp8_scale = fp8_scale
+    # upstream's kernels take alibi_slopes and softcap and ignore them; they act here only on request
+    if apply_alibi:
+        if alibi_slopes is None or alibi_slopes.dtype != torch.float32 or not alibi_slopes.is_contiguous() \
+                or alibi_slopes.numel() != H or alibi_slopes.device != query.device:
+            raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE, "apply_alibi needs contiguous fp32 alibi_slopes [num_heads] on the device")
+        op.mask_flags |= _cabi.FA_MASK_ALIBI
+    if apply_softcap:
+        op.mask_flags |= _cabi.FA_MASK_SOFTCAP
+    if window_left is not None:
+        op.mask_flags |= _cabi.FA_MASK_WINDOW
+        op.window_left = int(window_left)
     # bytes are E5M2 as upstream fixes them (paged_attention_fp8_loop.cpp:43) unless the tensor says E4M3
     op.kv_fp8_format = _cabi.FA_FP8_E4M3 if key_cache.dtype == torch.float8_e4m3fn else _cabi.FA_FP8_E5M2
     op.stream = torch.cuda.current_stream(query.device).cuda_stream

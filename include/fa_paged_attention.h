@@ -78,6 +78,13 @@ typedef enum fa_dtype { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 } fa_dtype;
  * no infinities, 0x7f / 0xff NaN. */
 typedef enum fa_fp8_format { FA_FP8_E5M2 = 0, FA_FP8_E4M3 = 1 } fa_fp8_format;
 
+/* Score modifiers upstream's kernels leave out (their code is commented out,
+ * paged_attention_kernel_loop.hpp:329-342) but upstream's test reference defines
+ * (test_paged.py:92-110), applied in its order: soft-capping softcap * tanh(s / softcap) of the
+ * scaled scores, the local window, then the ALiBi bias -alibi_slopes[h] * (distance to the
+ * query).  Opt-in: with mask_flags = 0 the entry points behave as upstream does. */
+typedef enum fa_mask { FA_MASK_ALIBI = 1, FA_MASK_SOFTCAP = 2, FA_MASK_WINDOW = 4 } fa_mask;
+
 /* Shapes and strides that upstream reads off the torch tensors
  * (paged_attention_loop.cpp:60-65) or fixes at compile time. */
 typedef struct fa_paged_attention_shape {
@@ -104,8 +111,8 @@ typedef struct fa_paged_attention_shape {
  * and timing control.  A NULL options pointer means all defaults. */
 typedef struct fa_paged_attention_options {
   const void *sinks;          /* device, [num_heads] in q_dtype, or NULL */
-  const float *alibi_slopes;  /* accepted, ignored */
-  float softcap;              /* accepted, ignored */
+  const float *alibi_slopes;  /* device, [num_heads] fp32; ignored unless FA_MASK_ALIBI */
+  float softcap;              /* ignored unless FA_MASK_SOFTCAP (then > 0) */
   float fp8_scale;            /* FP8 entries only: K^ = dequant(K)*s, V^ = dequant(V)*s; 0 means 1.0 */
   void *stream;               /* hipStream_t; NULL = the null stream */
   float *elapsed_us;          /* HOST pointer or NULL.  Non-NULL: the call synchronises and writes
@@ -115,6 +122,11 @@ typedef struct fa_paged_attention_options {
                                  launch_kernels_reduce.h:76-77).  NULL: asynchronous, no timing. */
   int32_t validate_only;      /* non-zero: check arguments, launch nothing */
   int32_t kv_fp8_format;      /* FP8 entries only: fa_fp8_format of the caches; 0 = E5M2 as upstream */
+  int32_t mask_flags;         /* bit set of fa_mask: which score modifiers to APPLY.  0, the default,
+                                 is upstream's behaviour: alibi_slopes and softcap are taken and
+                                 ignored */
+  int32_t window_left;        /* FA_MASK_WINDOW: the query (position context_len - 1) sees the keys
+                                 at positions context_len - 1 - window_left .. context_len - 1 */
 } fa_paged_attention_options;
 
 /* Single-pass kernel: one launch, no scratch. */

@@ -76,6 +76,8 @@ def lib() -> ctypes.CDLL:
         pp = ctypes.POINTER(_Problem)
         L.oracle_attention_ref.argtypes = [P, P, P, P, P, P, P, P, pp]
         L.oracle_attention_ref.restype = ctypes.c_int
+        L.oracle_attention_ref_masked.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32, pp]
+        L.oracle_attention_ref_masked.restype = ctypes.c_int
         L.oracle_kernel_loop.argtypes = [P, P, P, P, P, P, P, P, ctypes.c_int, pp]
         L.oracle_kernel_loop.restype = ctypes.c_int
         L.oracle_kernel_partition.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int, ctypes.c_int, pp]
@@ -146,16 +148,27 @@ def _bits_out(S, H, D, dtype):
 
 
 def attention_ref(query, key_cache, value_cache, block_tables, context_lens, *, scale, block_size,
-                  kv_strides, num_kv_heads, sinks=None, fp8_scale=1.0, want_f32=False):
-    """The upstream tests' PyTorch reference, restated (test_paged.py:40-168)."""
+                  kv_strides, num_kv_heads, sinks=None, fp8_scale=1.0, want_f32=False,
+                  alibi_slopes=None, softcap=0.0, window_left=-1):
+    """The upstream tests' PyTorch reference, restated (test_paged.py:40-168).  ``alibi_slopes``
+    ([heads] fp32), ``softcap`` > 0 and ``window_left`` >= 0 switch on the score modifiers of
+    test_paged.py:92-110."""
     pr = _problem(query, key_cache, value_cache, block_tables, context_lens, scale, block_size,
                   kv_strides, fp8_scale, num_kv_heads)
     S, H, D = query.shape
     out = torch.zeros((S, H, D), dtype=query.dtype)
     out32 = torch.zeros((S, H, D), dtype=torch.float32)
-    rc = lib().oracle_attention_ref(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
-                                    _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),
-                                    _ptr(sinks), ctypes.byref(pr))
+    if alibi_slopes is not None or softcap > 0 or window_left >= 0:
+        if alibi_slopes is not None:
+            assert alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and alibi_slopes.numel() == H
+        rc = lib().oracle_attention_ref_masked(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
+                                               _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),
+                                               _ptr(sinks), _ptr(alibi_slopes), float(softcap), int(window_left),
+                                               ctypes.byref(pr))
+    else:
+        rc = lib().oracle_attention_ref(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
+                                        _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),
+                                        _ptr(sinks), ctypes.byref(pr))
     if rc != 0:
         raise MemoryError("oracle_attention_ref")
     return (out, out32) if want_f32 else out

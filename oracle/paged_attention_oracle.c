@@ -37,6 +37,10 @@
  *                            split-invariance of log-sum-exp and by closed forms.
  *   e5m2 / e4m3 decode       pinned on all 256 codes against torch.float8_e5m2 /
  *                            torch.float8_e4m3fn.
+ *   oracle_attention_ref_masked  soft-capping, local window and ALiBi: pinned against SDPA
+ *                            with an additive bias / mask and against plain torch ops for
+ *                            the tanh cap (tests/test_oracle_masks.py).  Upstream's KERNELS
+ *                            do not implement these (the code is commented out there).
  *   fp8_scale != 1           PARITY UNPINNED: the upstream tests only ever pass
  *                            1.0 (test_paged_fp8cache.py:489,510); the reading
  *                            implemented is K^ = dequant(K)*s, V^ = dequant(V)*s.
@@ -228,10 +232,22 @@ CLONES static void axpy_f32(float *y, float a, const float *x, int n) {
  * sinks may be NULL; its entries are in the q dtype.
  * Returns 0, or -1 on allocation failure.
  */
-ORACLE_API int oracle_attention_ref(uint16_t *out, float *out_f32, const uint16_t *query,
-                                    const void *key_cache, const void *value_cache,
-                                    const int32_t *block_tables, const int32_t *context_lens,
-                                    const uint16_t *sinks, const oracle_problem *p) {
+/* The score modifiers of the upstream reference that its kernels leave out (commented-out
+ * code, paged_attention_kernel_loop.hpp:329-342) but its attention_ref defines
+ * (test_paged.py:92-110): soft-capping cap*tanh(s/cap) of the scaled scores, then the local
+ * window -- a decode query at position n-1 sees keys n-1-window_left .. n-1 -- then the
+ * ALiBi bias -slope_h * (n-1-t).  softcap <= 0, window_left < 0 and a NULL slope array each
+ * switch their modifier off. */
+typedef struct {
+  const float *alibi_slopes; /* [num_heads] or NULL */
+  float softcap;
+  int32_t window_left;
+} oracle_masks;
+
+static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *query,
+                              const void *key_cache, const void *value_cache,
+                              const int32_t *block_tables, const int32_t *context_lens,
+                              const uint16_t *sinks, const oracle_problem *p, const oracle_masks *mk) {
   const int S = p->num_seqs, H = p->num_heads, Hk = p->num_kv_heads, D = p->head_size;
   const int G = H / Hk;
   int failed = 0;
@@ -257,7 +273,11 @@ ORACLE_API int oracle_attention_ref(uint16_t *out, float *out_f32, const uint16_
           for (int d = 0; d < D; ++d) qf[d] = load16(qrow + d, p->q_dtype) * p->scale;
           float m = -INFINITY;
           for (int t = 0; t < n; ++t) {
-            sc[t] = dot_f32(qf, K + (size_t)t * D, D);
+            float x = dot_f32(qf, K + (size_t)t * D, D);
+            if (mk && mk->softcap > 0.f) x = mk->softcap * tanhf(x / mk->softcap);
+            if (mk && mk->window_left >= 0 && t < n - 1 - mk->window_left) x = -INFINITY;
+            if (mk && mk->alibi_slopes) x -= mk->alibi_slopes[h] * (float)(n - 1 - t);
+            sc[t] = x;
             if (sc[t] > m) m = sc[t];
           }
           float sink_term = 0.f;
@@ -285,6 +305,24 @@ ORACLE_API int oracle_attention_ref(uint16_t *out, float *out_f32, const uint16_
     }
   }
   return failed ? -1 : 0;
+}
+
+ORACLE_API int oracle_attention_ref(uint16_t *out, float *out_f32, const uint16_t *query,
+                                    const void *key_cache, const void *value_cache,
+                                    const int32_t *block_tables, const int32_t *context_lens,
+                                    const uint16_t *sinks, const oracle_problem *p) {
+  return attention_ref_core(out, out_f32, query, key_cache, value_cache, block_tables, context_lens,
+                            sinks, p, NULL);
+}
+
+ORACLE_API int oracle_attention_ref_masked(uint16_t *out, float *out_f32, const uint16_t *query,
+                                           const void *key_cache, const void *value_cache,
+                                           const int32_t *block_tables, const int32_t *context_lens,
+                                           const uint16_t *sinks, const float *alibi_slopes,
+                                           float softcap, int32_t window_left, const oracle_problem *p) {
+  oracle_masks mk = {alibi_slopes, softcap, window_left};
+  return attention_ref_core(out, out_f32, query, key_cache, value_cache, block_tables, context_lens,
+                            sinks, p, &mk);
 }
 
 /* ------------------------------------------------------------------ */

@@ -29,14 +29,15 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 2
+    assert L.fa_paged_attention_abi_version() == 3
 
 
 def test_struct_layouts_match_header():
     # field order and sizes of the two structs as the header lays them out
     assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
     assert _cabi.Shape.kv_block_stride.offset == 32
-    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4
+    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4
+    assert _cabi.Options.mask_flags.offset == 48 and _cabi.Options.window_left.offset == 52
     assert _cabi.Options.elapsed_us.offset == 32
     assert ctypes.sizeof(_cabi.KvWriteShape) == 4 * 4 + 5 * 8 + 2 * 4 + 8
     assert _cabi.KvWriteShape.src_dtype.offset == 56 and _cabi.KvWriteShape.num_pool_blocks.offset == 64
@@ -54,10 +55,12 @@ def _shape(**kw):
     return s
 
 
-def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0):
+def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0,
+          mask_flags=0, alibi=None, softcap=0.0, window_left=0):
     op = _cabi.Options()
     op.validate_only = 1
     op.kv_fp8_format = fp8_format
+    op.mask_flags, op.alibi_slopes, op.softcap, op.window_left = mask_flags, alibi, softcap, window_left
     name = "fa_paged_attention_" + ("fp8_" if fp8 else "") + ("reduce" if split else "loop")
     args = [ptr, ptr, ptr, ptr, ptr, ptr, 0.1, max_ctx]
     if split:
@@ -78,6 +81,17 @@ def test_fp8_format_is_checked_on_fp8_entries_only(L):
     assert _call(L, fp8=True, split=True, fp8_format=_cabi.FA_FP8_E4M3)[0] == _cabi.FA_OK
     assert _call(L, fp8=True, fp8_format=7)[0] == _cabi.FA_ERR_UNSUPPORTED_DTYPE
     assert _call(L, fp8=False, fp8_format=7)[0] == _cabi.FA_OK   # 16-bit entries ignore the field
+
+
+def test_score_modifier_arguments(L):
+    assert _call(L, mask_flags=0, softcap=-3.0, window_left=-9)[0] == _cabi.FA_OK      # ignored, as upstream
+    assert _call(L, mask_flags=_cabi.FA_MASK_ALIBI, alibi=0x1000)[0] == _cabi.FA_OK
+    assert _call(L, mask_flags=_cabi.FA_MASK_ALIBI)[0] == _cabi.FA_ERR_NULL_POINTER
+    assert _call(L, mask_flags=_cabi.FA_MASK_SOFTCAP, softcap=30.0)[0] == _cabi.FA_OK
+    assert _call(L, mask_flags=_cabi.FA_MASK_SOFTCAP, softcap=0.0)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _call(L, split=True, mask_flags=_cabi.FA_MASK_WINDOW, window_left=0)[0] == _cabi.FA_OK
+    assert _call(L, mask_flags=_cabi.FA_MASK_WINDOW, window_left=-1)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _call(L, mask_flags=8)[0] == _cabi.FA_ERR_BAD_SHAPE
 
 
 def test_error_codes(L):
