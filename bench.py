@@ -14,6 +14,7 @@ roofline     per-kernel HIP-event time on the launch stream (the library's own
 cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTorch
              reference) on the same workload on this box's host cores
 configs      the other four configurations, each timed the same way
+score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
              the asynchronous torch.library operators, and a HIP-graph replay of them
 kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
@@ -159,6 +160,34 @@ def _time_kv_cache_write(steps, torch, dev, cpu_leg):
     return res
 
 
+def _time_score_modifiers(built, steps, torch, W, runner, dev):
+    """Configuration 1 with the opt-in score modifiers: soft-capping 30, ALiBi, and a local window
+    of 1024 keys (the window shortens what has to be read; bytes are counted for visible keys)."""
+    from flash_attention_factory_amd.lib import paged_attention_loop
+    w, ks, vs = built
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    window_left = 1023
+    alibi = torch.linspace(0.002, 0.05, H, device=dev, dtype=torch.float32)
+    bufs = runner.alloc_buffers(w)
+    view = (lambda t: t.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR else (lambda t: t)
+    ts = []
+    for it in range(5 + steps):
+        k = it % len(ks)
+        t = paged_attention_loop.run(None, None, None, bufs.out, None, w.query, view(ks[k]), view(vs[k]),
+                                     w.block_tables, w.context_lens, H // Hk, w.scale, B, 0, alibi, w.sinks, 30.0,
+                                     apply_alibi=True, apply_softcap=True, window_left=window_left)
+        if it >= 5:
+            ts.append(t[0])
+    us = float(torch.tensor(ts, dtype=torch.float64).mean())
+    visible = torch.clamp(w.context_lens, max=window_left + 1).sum().item()
+    nbytes = visible * Hk * D * 2 * w.key_cache.element_size() + 2 * S * H * D * 2 + 4 * S + 4 * H \
+        + sum(-(-min(int(c), window_left + 1) // B) for c in w.context_lens.tolist()) * 4
+    return dict(workload="config1 + soft-capping 30 + ALiBi + local window of 1024 keys (grid-form kernel)",
+                kernel="paged_attn_kernel<128, F16, kv16, loop, modifiers>", steps=steps, us_per_call=us,
+                algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
+
+
 def _time_stream_ordered(steps, torch, W, runner, dev):
     """Host cost of one small decode step (configuration 0: KV-cache append of one token per
     sequence, then the loop kernel) three ways: the timed `run` calls, which block on every
@@ -276,6 +305,7 @@ def main():
                      "kernel_us": kernel_us},
         "configs": others,
     }
+    line["score_modifiers"] = _time_score_modifiers(built[1], max(20, args.steps // 2), torch, W, runner, dev)
     # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
     e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
     _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
