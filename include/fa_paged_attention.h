@@ -41,7 +41,8 @@
  * h / (num_heads / num_kv_heads); tokens at or beyond context_lens[s] never
  * contribute; an optional per-head sink logit joins the softmax denominator only;
  * alibi_slopes and softcap are accepted and ignored exactly as upstream
- * (paged_attention_kernel_loop.hpp:175-178,329-342 are commented out there).
+ * (paged_attention_kernel_loop.hpp:175-178,329-342 are commented out there) unless
+ * options->mask_flags asks for them (see fa_mask below).
  * A sequence with context_lens[s] <= 0 leaves its rows of `out` untouched; a
  * context length above max_blocks_per_seq * block_size is cut to that bound, so the
  * kernels never read past a row of block_tables.
