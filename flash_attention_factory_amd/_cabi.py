@@ -75,6 +75,8 @@ class Options(ctypes.Structure):
         ("kv_fp8_format", ctypes.c_int32),
         ("mask_flags", ctypes.c_int32),
         ("window_left", ctypes.c_int32),
+        ("query_len", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 

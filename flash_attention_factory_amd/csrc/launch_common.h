@@ -59,6 +59,7 @@ struct Resolved {
   const float *alibi_slopes;
   float softcap;
   int32_t window_left;
+  int32_t query_len;  // query tokens per sequence, >= 1
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -138,6 +139,14 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
     return fail(FA_ERR_BAD_SHAPE, "FA_MASK_SOFTCAP needs softcap > 0");
   if ((r->mask_flags & FA_MASK_WINDOW) && o->window_left < 0)
     return fail(FA_ERR_BAD_SHAPE, "FA_MASK_WINDOW needs window_left >= 0");
+  r->query_len = (o && o->query_len > 1) ? o->query_len : 1;
+  if (o && o->query_len < 0) return fail(FA_ERR_BAD_SHAPE, "query_len must be >= 0");
+  if ((int64_t)r->query_len * r->group > kMaxGroup)
+    return fail(FA_ERR_UNSUPPORTED_GROUP, "query_len %d x %d queries per kv head exceeds %d", r->query_len,
+                r->group, kMaxGroup);
+  if ((int64_t)s->num_seqs * r->query_len > 65535)
+    return fail(FA_ERR_BAD_SHAPE, "num_seqs x query_len %lld exceeds the grid limit 65535",
+                (long long)s->num_seqs * r->query_len);
   r->alibi_slopes = o ? o->alibi_slopes : nullptr;
   r->softcap = o ? o->softcap : 0.f;
   r->window_left = o ? o->window_left : 0;
@@ -169,6 +178,7 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.alibi_slopes = r.alibi_slopes;
   p.softcap = r.softcap;
   p.window_left = r.window_left;
+  p.query_len = r.query_len;
   p.out_scale = r.fp8_scale;
   p.num_seqs = s.num_seqs;
   p.num_heads = s.num_heads;

@@ -28,8 +28,8 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
   const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
-  if (r.mask_flags != 0) {
-    // score modifiers: the grid form has the instance that applies them
+  if (r.mask_flags != 0 || r.query_len > 1) {
+    // score modifiers, several query tokens: the grid form has the instance for them
     const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
         paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,

@@ -32,8 +32,8 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // work-group per (kv head, partition slot, sequence); slots past a sequence's length
   // return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
   int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
-  if (r.mask_flags != 0) {
-    // score modifiers: the grid form has the instance that applies them
+  if (r.mask_flags != 0 || r.query_len > 1) {
+    // score modifiers, several query tokens: the grid form has the instance for them
     const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
         paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
@@ -72,9 +72,10 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
   rp.num_seqs = shape.num_seqs;
   rp.num_kv_heads = shape.num_kv_heads;
+  rp.query_len = r.query_len;
   rp.segment_groups = segment_groups;
-  const dim3 rgrid(shape.num_heads, shape.num_seqs);
-  const bool one_wave = (int64_t)shape.num_heads * shape.num_seqs >= kReduceSingleWaveMinPairs;
+  const dim3 rgrid(shape.num_heads, shape.num_seqs * r.query_len);
+  const bool one_wave = (int64_t)shape.num_heads * shape.num_seqs * r.query_len >= kReduceSingleWaveMinPairs;
   if (segment_groups > 0) {
     if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, true>, rgrid, dim3(64), 1, rp));
     else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, true>, rgrid, dim3(256), 1, rp));

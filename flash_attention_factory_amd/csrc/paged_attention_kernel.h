@@ -71,31 +71,32 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
     }
   }
 
-  if (i >= p.group) return;
-  const float inv = L > 0.f ? p.out_scale / L : 0.f;  // L = 0: a partition wholly before a local window
-  const int head = kvh * p.group + i;
+  if (!wa.col_valid) return;
+  const float inv = L > 0.f ? p.out_scale / L : 0.f;  // L = 0: nothing visible (local window, causal rule)
+  const int head = kvh * p.group + wa.col_g;
+  const int64_t row = W::kExt ? (int64_t)seq * p.query_len + wa.col_q : seq;  // row of query / out / scratch
   const int d0 = 4 * r * NDT + wave * SL;  // first head-dim element this lane stores
   if constexpr (PART) {
-    const int64_t slot = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions + part;
+    const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part;
     W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
     if (r == 0 && wave == 0) {
       p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
       p.exp_sums[slot] = L;
     }
   } else {
-    W::template store_q<SL>(reinterpret_cast<char *>(p.out) +
-                                (((int64_t)seq * p.num_heads + head) * D + d0) * 2,
-                            o, inv);
+    W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
   }
 }
 
-// MASKS: an instance that also applies the score modifiers of p.mask_flags (soft-capping,
-// local window, ALiBi).  Chunks that lie wholly before a sequence's window are skipped; a
-// partition that lies wholly before it stores an empty partial (max -inf, sum 0, zeros).
+// MASKS: the extended instance.  It applies the score modifiers of p.mask_flags (soft-capping,
+// local window, ALiBi) and takes p.query_len query tokens per sequence, causal among
+// themselves (speculative decoding, chunked prefill): the MFMA columns are then (query token,
+// head) pairs.  Chunks that lie wholly before a sequence's window are skipped; a partition
+// of which a column sees nothing stores an empty partial for it (max -inf, sum 0, zeros).
 template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC, bool MASKS = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop>;
+  using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop, MASKS>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;
@@ -132,7 +133,9 @@ paged_attn_kernel(const PagedAttnParams p) {
   int c_lo = c_begin;  // first chunk that holds a visible token
   if constexpr (MASKS) {
     wa.load_slope(kvh);
-    if (p.mask_flags & kMaskWindow) c_lo = max(c_begin, max(0, ctx - 1 - p.window_left) / CT);
+    wa.set_context(ctx);
+    // the earliest query token's window decides where reading starts
+    if (p.mask_flags & kMaskWindow) c_lo = max(c_begin, max(0, ctx - p.query_len - p.window_left) / CT);
   }
 
   // ---- streaming loop ------------------------------------------------------------------
@@ -155,14 +158,14 @@ paged_attn_kernel(const PagedAttnParams p) {
       const int cn = ci + NW;
       const auto s = wa.qk(R);
       wa.issue_k(R, kvh, cn, nids);
-      const auto pb = wa.template soft<false, MASKS>(R, s, ci, tok_end, ctx - 1);
+      const auto pb = wa.template soft<false, MASKS>(R, s, ci, tok_end);
       wa.pv(R, pb);
       wa.issue_v(R, kvh, cn, nids);
       nids = wa.fetch_ids(table, cn + NW, last_blk);
       ci = cn;
     }
     const auto s = wa.qk(R);
-    wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end, ctx - 1));
+    wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end));
   }
 
   merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part);

@@ -35,6 +35,7 @@ struct ReduceParams {
   int32_t max_context;  // max_blocks_per_seq * block_size: lengths are cut to it
   int32_t num_seqs;
   int32_t num_kv_heads;
+  int32_t query_len;       // query tokens per sequence: rows of out / scratch are (sequence, query token) pairs
   int32_t segment_groups;  // work-groups of the segment attention kernel that wrote the partials
                            // (it wrote one partial per segment of m partitions, into the
                            // segment's first slot); 0: one partial per partition
@@ -57,8 +58,8 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int head = blockIdx.x;
-  const int seq = blockIdx.y;
-  const int ctx = min(p.context_lens[seq], p.max_context);
+  const int seq = blockIdx.y;  // row of out and of the scratch arrays
+  const int ctx = min(p.context_lens[p.query_len > 1 ? seq / p.query_len : seq], p.max_context);
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;
   np = min(np, p.max_num_partitions);

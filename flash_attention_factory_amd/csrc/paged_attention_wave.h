@@ -54,6 +54,7 @@ struct PagedAttnParams {
   float softcap;
   int32_t window_left;
   int32_t mask_flags;           // kMaskAlibi | kMaskSoftcap | kMaskWindow
+  int32_t query_len;            // query tokens per sequence (1 = plain decode)
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
@@ -61,9 +62,13 @@ constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask o
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
 // KVF: cache format, kKv16 (elements of the query type), kKvE5M2 or kKvE4M3 (bytes).
-template <int D, typename QT, int KVF, int TPC, bool STREAM>
+// EXT: the extended instance -- score modifiers and several query tokens per sequence
+// (p.mask_flags, p.query_len).  The MFMA columns then stand for (query token, head) pairs:
+// column i = query token i / G, head i % G of the kv head's group.
+template <int D, typename QT, int KVF, int TPC, bool STREAM, bool EXT = false>
 struct WaveAttn {
   static constexpr bool KV8 = KVF != kKv16;
+  static constexpr bool kExt = EXT;
   static_assert(TPC == 2 || TPC == 4, "a chunk is one or two 32-token P.V steps");
   static constexpr int ROWB = D * (KV8 ? 1 : 2);  // bytes per token row
   static constexpr int KL = ROWB / 64;            // 16-byte K loads per lane and tile
@@ -89,6 +94,9 @@ struct WaveAttn {
   const int r;  // 16-lane row of the wavefront
   const int i;  // position in the row: token (K), head (Q, P, O) or d-row (V)
   const int blk_mask;
+  // EXT only: what column i stands for, and the position of its query token
+  int col_q = 0, col_g = 0, col_last = 0;
+  bool col_valid = false;
 
   // Q^T as the MFMA "B" operand, one dword quad per k-step.  k-slot (r, e) of step c
   // stands for head-dim element qd(c, r) + e; K uses the same map.
@@ -101,22 +109,35 @@ struct WaveAttn {
   float slope_log2 = 0.f;  // ALiBi slope of head i in base-2 units (MASKS instances only)
 
   __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
-      : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {}
+      : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {
+    if constexpr (EXT) {
+      col_q = i / prm.group;
+      col_g = i - col_q * prm.group;
+      col_valid = i < prm.group * prm.query_len;
+    } else {
+      col_g = i;
+      col_valid = i < prm.group;
+    }
+  }
+
+  // EXT: the context length of the item at hand; query token q sits at position
+  // ctx - query_len + q and sees the keys up to there.
+  __device__ __forceinline__ void set_context(int ctx) { col_last = ctx - p.query_len + col_q; }
 
   // ALiBi slope of this lane's head; kernels built with MASKS call it once per item.
   __device__ __forceinline__ void load_slope(int kvh) {
-    slope_log2 = ((p.mask_flags & kMaskAlibi) && i < p.group) ? p.alibi_slopes[kvh * p.group + i] * kLog2e : 0.f;
+    slope_log2 = ((p.mask_flags & kMaskAlibi) && col_valid) ? p.alibi_slopes[kvh * p.group + col_g] * kLog2e : 0.f;
   }
 
   __device__ __forceinline__ void load_q(int seq, int kvh) {
-    const int head = kvh * p.group + i;
-    const char *qrow = reinterpret_cast<const char *>(p.query) +
-                       ((int64_t)seq * p.num_heads + head) * (D * 2);
+    const int head = kvh * p.group + col_g;
+    const int64_t row = EXT ? (int64_t)seq * p.query_len + col_q : seq;
+    const char *qrow = reinterpret_cast<const char *>(p.query) + (row * p.num_heads + head) * (D * 2);
 #pragma unroll
     for (int c = 0; c < KSTEPS; ++c) {
       const int d0 = KV8 ? ((c >> 1) * 4 + r) * 16 + (c & 1) * 8 : (c * 4 + r) * 8;
       u32x4 z = {0u, 0u, 0u, 0u};
-      qB[c] = (i < p.group) ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
+      qB[c] = col_valid ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
     }
   }
 
@@ -128,9 +149,9 @@ struct WaveAttn {
   static constexpr uint32_t kNoSink = 0xffffffffu;
   __device__ __forceinline__ uint32_t load_sink(int kvh, bool with_sink) const {
     uint32_t raw = kNoSink;
-    if (with_sink && p.sinks != nullptr && i < p.group)
+    if (with_sink && p.sinks != nullptr && col_valid)
       raw = *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(p.sinks) +
-                                                (kvh * p.group + i) * 2);
+                                                (kvh * p.group + col_g) * 2);
     return raw;
   }
 
@@ -236,17 +257,17 @@ struct WaveAttn {
   // Online softmax step over the chunk's tokens; returns the P^T "B" operands.
   // check_tail: whether this chunk can reach past tok_end (a compile-time false drops
   // the masking code from the steady-state loop).
-  // MASKS: apply the score modifiers p.mask_flags names -- soft-capping, local window, ALiBi,
-  // in that order (upstream test_paged.py:92-110) -- for a query at position `last_pos`.
-  // The caller never hands over a chunk that lies wholly before the window.
+  // MASKS (EXT instances): apply the score modifiers p.mask_flags names -- soft-capping, local
+  // window, ALiBi, in that order (upstream test_paged.py:92-110) -- and the causal rule, all
+  // relative to the position col_last of this column's query token.
   template <bool CHECK_TAIL, bool MASKS = false>
-  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end, int last_pos = 0) {
+  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
     float t[NT];
     if constexpr (MASKS) {
       const bool cap = p.mask_flags & kMaskSoftcap;
       const float inv_cap2 = 2.0f * kLog2e / p.softcap;  // exp(2x/cap) = exp2(x * inv_cap2)
-      const int first_visible = (p.mask_flags & kMaskWindow) ? last_pos - p.window_left : 0;
+      const int first_visible = (p.mask_flags & kMaskWindow) ? col_last - p.window_left : 0;
 #pragma unroll
       for (int e = 0; e < NT; ++e) {
         float x = s.v[e >> 2][e & 3] * p.score_scale;
@@ -255,8 +276,8 @@ struct WaveAttn {
           x = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f));
         }
         const int tok = ci * CT + (e >> 2) * kTileTokens + 4 * r + (e & 3);
-        x = x * kLog2e + slope_log2 * (float)(tok - last_pos);
-        t[e] = tok < first_visible ? -INFINITY : x;
+        x = x * kLog2e + slope_log2 * (float)(tok - col_last);
+        t[e] = (tok < first_visible || tok > col_last) ? -INFINITY : x;
       }
     } else {
 #pragma unroll
@@ -281,11 +302,14 @@ struct WaveAttn {
     for (int e = 1; e < NT; ++e) mx = fmaxf(mx, t[e]);
     mx = rows_max(mx);
     const float m_new = fmaxf(m, mx);
-    const float alpha = fast_exp2(m - m_new);  // exp2(-inf) = 0 on the first chunk
+    // MASKS: a column may see nothing of a chunk (a query token before the chunk's keys)
+    // and nothing before it either; subtract 0 then, so that -inf stays -inf, not NaN
+    const float m_sub = (MASKS && m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_sub);  // exp2(-inf) = 0 on the first chunk
     float ps = 0.f;
 #pragma unroll
     for (int e = 0; e < NT; ++e) {
-      t[e] = fast_exp2(t[e] - m_new);
+      t[e] = fast_exp2(t[e] - m_sub);
       ps += t[e];
     }
     l = l * alpha + ps;

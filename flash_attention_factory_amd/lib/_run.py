@@ -23,8 +23,10 @@ _scratch = {}
 def _fp32_scratch(tem_output: torch.Tensor, shape) -> torch.Tensor:
     """Upstream keeps tem_output in the query dtype; the kernels here want fp32.  A
     caller that passes a 16-bit tem_output gets a cached fp32 workspace instead."""
-    if tem_output.dtype == torch.float32 and tuple(tem_output.shape) == tuple(shape) \
-            and tem_output.is_contiguous():
+    want = 1
+    for n in shape:
+        want *= n
+    if tem_output.dtype == torch.float32 and tem_output.numel() == want and tem_output.is_contiguous():
         return tem_output
     key = (tem_output.device, tuple(shape))
     buf = _scratch.get(key)
@@ -62,13 +64,19 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
                                         "caches must be 4-D [blocks, block_size, kv_heads, head_size] "
                                         "views with a contiguous last dimension and equal strides")
-    S, H, D = query.shape
+    # [S, H, D], or [S, query_len, H, D]: several query tokens per sequence (causal among themselves)
+    if query.dim() == 4:
+        S, QL, H, D = query.shape
+    else:
+        (S, H, D), QL = query.shape, 1
+    if output.shape != query.shape:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE, "output must have the shape of query")
     sh = _cabi.Shape()
     sh.num_seqs, sh.num_heads, sh.head_size = S, H, D
     sh.num_kv_heads = key_cache.size(2)
     sh.block_size = block_size
     sh.max_blocks_per_seq = block_tables.size(1)
-    sh.max_num_partitions = max_logits.size(2) if split else 1
+    sh.max_num_partitions = max_logits.size(-1) if split else 1
     sh.partition_size = partition_size
     sh.kv_block_stride, sh.kv_token_stride, sh.kv_head_stride = (
         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
@@ -97,6 +105,7 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     if window_left is not None:
         op.mask_flags |= _cabi.FA_MASK_WINDOW
         op.window_left = int(window_left)
+    op.query_len = QL
     # bytes are E5M2 as upstream fixes them (paged_attention_fp8_loop.cpp:43) unless the tensor says E4M3
     op.kv_fp8_format = _cabi.FA_FP8_E4M3 if key_cache.dtype == torch.float8_e4m3fn else _cabi.FA_FP8_E5M2
     op.stream = torch.cuda.current_stream(query.device).cuda_stream
@@ -105,7 +114,10 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     args = [output.data_ptr(), query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
             block_tables.data_ptr(), context_lens.data_ptr(), float(sm_scale), int(max_context_len)]
     if split:
-        tmp = _fp32_scratch(tem_output, (S, H, sh.max_num_partitions, D))
+        tmp = _fp32_scratch(tem_output, (S * QL, H, sh.max_num_partitions, D))
+        if max_logits.numel() != S * QL * H * sh.max_num_partitions or exp_sums.numel() != max_logits.numel():
+            raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
+                                            "max_logits/exp_sums must hold [num_seqs * query_len, num_heads, partitions]")
         if max_logits.dtype != torch.float32 or exp_sums.dtype != torch.float32 \
                 or not max_logits.is_contiguous() or not exp_sums.is_contiguous():
             raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE,

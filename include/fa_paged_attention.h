@@ -128,6 +128,15 @@ typedef struct fa_paged_attention_options {
                                  ignored */
   int32_t window_left;        /* FA_MASK_WINDOW: the query (position context_len - 1) sees the keys
                                  at positions context_len - 1 - window_left .. context_len - 1 */
+  int32_t query_len;          /* query tokens per sequence; 0 or 1 = decode.  With n > 1 (speculative
+                                 decoding, chunked prefill) query and out are
+                                 [num_seqs, n, num_heads, head_size], the scratch arrays have
+                                 num_seqs * n rows, the n tokens are the last n positions of the
+                                 context (their K/V rows already in the caches, context_lens counting
+                                 them) and token j sees the keys up to its own position -- upstream's
+                                 causal rule, test_paged.py:79-80.  n * (num_heads / num_kv_heads)
+                                 must not exceed 16 */
+  int32_t reserved;
 } fa_paged_attention_options;
 
 /* Single-pass kernel: one launch, no scratch. */

@@ -76,7 +76,8 @@ def lib() -> ctypes.CDLL:
         pp = ctypes.POINTER(_Problem)
         L.oracle_attention_ref.argtypes = [P, P, P, P, P, P, P, P, pp]
         L.oracle_attention_ref.restype = ctypes.c_int
-        L.oracle_attention_ref_masked.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32, pp]
+        L.oracle_attention_ref_masked.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32,
+                                                  ctypes.c_int32, pp]
         L.oracle_attention_ref_masked.restype = ctypes.c_int
         L.oracle_kernel_loop.argtypes = [P, P, P, P, P, P, P, P, ctypes.c_int, pp]
         L.oracle_kernel_loop.restype = ctypes.c_int
@@ -153,18 +154,24 @@ def attention_ref(query, key_cache, value_cache, block_tables, context_lens, *, 
     """The upstream tests' PyTorch reference, restated (test_paged.py:40-168).  ``alibi_slopes``
     ([heads] fp32), ``softcap`` > 0 and ``window_left`` >= 0 switch on the score modifiers of
     test_paged.py:92-110."""
-    pr = _problem(query, key_cache, value_cache, block_tables, context_lens, scale, block_size,
+    query_len = 1
+    q3 = query
+    if query.dim() == 4:  # [S, query_len, H, D]: several query tokens per sequence, causal among themselves
+        query_len = query.shape[1]
+        q3 = query.reshape(query.shape[0] * query_len, query.shape[2], query.shape[3])
+    pr = _problem(q3, key_cache, value_cache, block_tables, context_lens, scale, block_size,
                   kv_strides, fp8_scale, num_kv_heads)
-    S, H, D = query.shape
-    out = torch.zeros((S, H, D), dtype=query.dtype)
-    out32 = torch.zeros((S, H, D), dtype=torch.float32)
-    if alibi_slopes is not None or softcap > 0 or window_left >= 0:
+    pr.num_seqs = query.shape[0]
+    S, H, D = q3.shape
+    out = torch.zeros(query.shape, dtype=query.dtype)
+    out32 = torch.zeros(query.shape, dtype=torch.float32)
+    if alibi_slopes is not None or softcap > 0 or window_left >= 0 or query_len > 1:
         if alibi_slopes is not None:
             assert alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and alibi_slopes.numel() == H
         rc = lib().oracle_attention_ref_masked(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
                                                _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),
                                                _ptr(sinks), _ptr(alibi_slopes), float(softcap), int(window_left),
-                                               ctypes.byref(pr))
+                                               int(query_len), ctypes.byref(pr))
     else:
         rc = lib().oracle_attention_ref(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
                                         _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),

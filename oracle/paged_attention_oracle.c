@@ -242,6 +242,13 @@ typedef struct {
   const float *alibi_slopes; /* [num_heads] or NULL */
   float softcap;
   int32_t window_left;
+  int32_t query_len; /* query tokens per sequence (speculative decoding, chunked prefill):
+                        query and out are [num_seqs, query_len, num_heads, head_size]; the
+                        query tokens are the LAST query_len positions of the context (their
+                        K/V rows are in the cache) and each sees the keys up to its own
+                        position -- upstream's causal rule, key j visible to query i iff
+                        j <= i + seqlen_k - seqlen_q (test_paged.py:79-80 with the local mask
+                        of :98-109).  1 = plain decode. */
 } oracle_masks;
 
 static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *query,
@@ -254,22 +261,26 @@ static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *que
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
   for (int s = 0; s < S; ++s) {
     for (int kh = 0; kh < Hk; ++kh) {
-      const int n = context_lens[s];
-      if (n <= 0) continue;
-      float *K = (float *)malloc((size_t)n * D * sizeof(float));
-      float *V = (float *)malloc((size_t)n * D * sizeof(float));
-      float *sc = (float *)malloc((size_t)n * sizeof(float));
+      const int n_all = context_lens[s];
+      const int QL = mk && mk->query_len > 1 ? mk->query_len : 1;
+      if (n_all <= 0) continue;
+      float *K = (float *)malloc((size_t)n_all * D * sizeof(float));
+      float *V = (float *)malloc((size_t)n_all * D * sizeof(float));
+      float *sc = (float *)malloc((size_t)n_all * sizeof(float));
       float *qf = (float *)malloc((size_t)D * sizeof(float));
       float *acc = (float *)malloc((size_t)D * sizeof(float));
       if (!K || !V || !sc || !qf || !acc) {
         failed = 1;
       } else {
         const int32_t *table = block_tables + (size_t)s * p->max_blocks_per_seq;
-        gather_rows(K, key_cache, table, n, kh, p);
-        gather_rows(V, value_cache, table, n, kh, p);
-        for (int g = 0; g < G; ++g) {
+        gather_rows(K, key_cache, table, n_all, kh, p);
+        gather_rows(V, value_cache, table, n_all, kh, p);
+        for (int qg = 0; qg < QL * G; ++qg) {
+          const int qt = qg / G, g = qg % G;
+          const int n = n_all - QL + qt + 1; /* keys this query token sees */
+          if (n <= 0) continue;
           const int h = kh * G + g;
-          const uint16_t *qrow = query + ((size_t)s * H + h) * D;
+          const uint16_t *qrow = query + (((size_t)s * QL + qt) * H + h) * D;
           for (int d = 0; d < D; ++d) qf[d] = load16(qrow + d, p->q_dtype) * p->scale;
           float m = -INFINITY;
           for (int t = 0; t < n; ++t) {
@@ -294,7 +305,7 @@ static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *que
           denom += sink_term;
           for (int d = 0; d < D; ++d) acc[d] = 0.f;
           for (int t = 0; t < n; ++t) axpy_f32(acc, sc[t] / denom, V + (size_t)t * D, D);
-          size_t o = ((size_t)s * H + h) * D;
+          size_t o = (((size_t)s * QL + qt) * H + h) * D;
           for (int d = 0; d < D; ++d) {
             if (out_f32) out_f32[o + d] = acc[d];
             if (out) out[o + d] = round16(acc[d], p->q_dtype);
@@ -319,8 +330,9 @@ ORACLE_API int oracle_attention_ref_masked(uint16_t *out, float *out_f32, const 
                                            const void *key_cache, const void *value_cache,
                                            const int32_t *block_tables, const int32_t *context_lens,
                                            const uint16_t *sinks, const float *alibi_slopes,
-                                           float softcap, int32_t window_left, const oracle_problem *p) {
-  oracle_masks mk = {alibi_slopes, softcap, window_left};
+                                           float softcap, int32_t window_left, int32_t query_len,
+                                           const oracle_problem *p) {
+  oracle_masks mk = {alibi_slopes, softcap, window_left, query_len};
   return attention_ref_core(out, out_f32, query, key_cache, value_cache, block_tables, context_lens,
                             sinks, p, &mk);
 }

@@ -29,14 +29,15 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 3
+    assert L.fa_paged_attention_abi_version() == 4
 
 
 def test_struct_layouts_match_header():
     # field order and sizes of the two structs as the header lays them out
     assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
     assert _cabi.Shape.kv_block_stride.offset == 32
-    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4
+    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4
+    assert _cabi.Options.query_len.offset == 56
     assert _cabi.Options.mask_flags.offset == 48 and _cabi.Options.window_left.offset == 52
     assert _cabi.Options.elapsed_us.offset == 32
     assert ctypes.sizeof(_cabi.KvWriteShape) == 4 * 4 + 5 * 8 + 2 * 4 + 8
@@ -56,8 +57,9 @@ def _shape(**kw):
 
 
 def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0,
-          mask_flags=0, alibi=None, softcap=0.0, window_left=0):
+          mask_flags=0, alibi=None, softcap=0.0, window_left=0, query_len=0):
     op = _cabi.Options()
+    op.query_len = query_len
     op.validate_only = 1
     op.kv_fp8_format = fp8_format
     op.mask_flags, op.alibi_slopes, op.softcap, op.window_left = mask_flags, alibi, softcap, window_left
@@ -92,6 +94,13 @@ def test_score_modifier_arguments(L):
     assert _call(L, split=True, mask_flags=_cabi.FA_MASK_WINDOW, window_left=0)[0] == _cabi.FA_OK
     assert _call(L, mask_flags=_cabi.FA_MASK_WINDOW, window_left=-1)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _call(L, mask_flags=8)[0] == _cabi.FA_ERR_BAD_SHAPE
+
+
+def test_query_len_limits(L):
+    assert _call(L, query_len=4)[0] == _cabi.FA_OK                      # group 4 x 4 tokens = 16 columns
+    assert _call(L, query_len=5)[0] == _cabi.FA_ERR_UNSUPPORTED_GROUP
+    assert _call(L, split=True, query_len=2)[0] == _cabi.FA_OK
+    assert _call(L, query_len=-1)[0] == _cabi.FA_ERR_BAD_SHAPE
 
 
 def test_error_codes(L):

@@ -87,3 +87,71 @@ def test_default_ignores_slopes_and_cap(oracle):
     for kernel in ("loop", "reduce"):
         got = _call(wd, kernel, alibi_slopes=ones, softcap=3.0).float().cpu()
         torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL)
+
+
+def _call_multi(w, query4, kernel, **mods):
+    """lib.<kernel>.run with query/out of shape [S, query_len, H, D] and scratch rows to match."""
+    dev = query4.device
+    mod = getattr(lib, "paged_attention_" + kernel)
+    S, QL, H, D = query4.shape
+    Hk = w.num_kv_heads
+    NP = -(-int(w.context_lens.max()) // w.partition_size)
+    out = torch.zeros_like(query4)
+    ml = torch.full((S * QL, H, NP), float("nan"), dtype=torch.float32, device=dev)
+    es = torch.full_like(ml, float("nan"))
+    tmp = torch.full((S * QL, H, NP, D), float("nan"), dtype=torch.float32, device=dev)
+    kv, vv = (w.key_cache.permute(0, 2, 1, 3), w.value_cache.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR \
+        else (w.key_cache, w.value_cache)
+    head = [ml, es, tmp, out, None, query4, kv, vv, w.block_tables, w.context_lens, H // Hk, w.scale]
+    if kernel.startswith("fp8"):
+        head.append(w.fp8_scale)
+    alibi, softcap = mods.pop("alibi_slopes", None), mods.pop("softcap", 0.0)
+    extra = dict(partition_size=w.partition_size) if "reduce" in kernel else {}
+    mod.run(*head, w.block_size, int(w.context_lens.max()), alibi, w.sinks, softcap, **extra, **mods)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("QL,nheads,nheads_k", [(2, 8, 2), (4, 8, 2), (8, 4, 2), (16, 2, 2), (3, 10, 2)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_several_query_tokens_per_sequence(oracle, QL, nheads, nheads_k, fp8):
+    """Speculative-decoding shaped calls: QL query tokens per sequence, causal among themselves,
+    (query token, head) pairs filling the 16 MFMA columns."""
+    w = W.make_test_shaped(batch_size=4, nheads=nheads, nheads_k=nheads_k, d=128, seqlen_k=1400, varlen=True,
+                           has_sinks=True, fp8=fp8, seed=13)
+    w.context_lens[0] = QL                 # the query tokens are the whole context
+    w.context_lens[1] = 512 + 1            # the last query token opens a new partition
+    w.context_lens[2] = 1024               # the query tokens end exactly on a partition boundary
+    g = torch.Generator().manual_seed(4)
+    query4 = torch.randn(4, QL, nheads, 128, generator=g).to(torch.float16)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, fp8_scale=w.fp8_scale, want_f32=True)[1]
+    wd = w.to(_dev())
+    for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+        got = _call_multi(wd, query4.to(_dev()), kernel).float().cpu()
+        assert torch.isfinite(got).all(), kernel
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel} QL={QL}: {m}")
+
+
+def test_query_tokens_with_modifiers_and_last_token_equals_decode(oracle):
+    w = W.make_config(4, num_seqs=3, pool_blocks=1200, lens=[3000, 70, 1537])      # bf16, E5M2, G = 8
+    H = w.query.shape[1]
+    QL = 2
+    g = torch.Generator().manual_seed(6)
+    query4 = torch.randn(3, QL, H, 128, generator=g).to(torch.bfloat16)
+    alibi = torch.linspace(0.001, 0.02, H)
+    okw = dict(alibi_slopes=alibi, softcap=25.0, window_left=900)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               fp8_scale=w.fp8_scale, want_f32=True, **okw)[1]
+    wd = w.to(_dev())
+    mods = dict(alibi_slopes=alibi.to(_dev()), softcap=25.0, apply_alibi=True, apply_softcap=True, window_left=900)
+    for kernel in ("fp8_loop", "fp8_reduce"):
+        got = _call_multi(wd, query4.to(_dev()), kernel, **dict(mods))
+        torch.testing.assert_close(got.float().cpu(), ref, atol=ATOL, rtol=RTOL)
+        # the last query token alone is a plain decode call with the same modifiers
+        wq = W.Workload(**{**wd.__dict__})
+        wq.query = query4[:, -1].contiguous().to(_dev())
+        single = _call(wq, kernel, **dict(mods))
+        torch.testing.assert_close(got[:, -1].float(), single.float(), atol=2e-3, rtol=2e-2)

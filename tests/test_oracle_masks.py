@@ -65,3 +65,52 @@ def test_masked_attention_ref_matches_torch(oracle, mk, sinks, fp8):
         assert not torch.equal(got, plain)   # the bias acts although the window does not
     if mk == dict(window_left=0):            # only the last key is visible: out = its value row, sink-weighted
         assert torch.isfinite(got).all()
+
+
+def _reference_multi(w, query4, alibi=None, window_left=-1):
+    """SDPA over [S, H, QL, T] with the causal rule of upstream's reference: the QL query tokens
+    are the last QL positions and token j of them sees keys 0 .. n - QL + j."""
+    S, QL, H, D = query4.shape
+    G = H // w.num_kv_heads
+    k = (dense_kv(w, w.key_cache) * w.fp8_scale).repeat_interleave(G, dim=2).permute(0, 2, 1, 3)
+    v = (dense_kv(w, w.value_cache) * w.fp8_scale).repeat_interleave(G, dim=2).permute(0, 2, 1, 3)
+    T = k.shape[2]
+    q = query4.float().permute(0, 2, 1, 3)                                   # [S, H, QL, D]
+    pos = torch.arange(T)[None, None, :]
+    last = (w.context_lens[:, None].long() - QL + torch.arange(QL)[None, :])[:, :, None]   # [S, QL, 1]
+    dead = pos > last
+    if window_left >= 0:
+        dead = dead | (pos < last - window_left)
+    bias = torch.zeros(S, 1, QL, T).masked_fill(dead[:, None], float("-inf")).expand(S, H, QL, T).clone()
+    if alibi is not None:
+        bias = bias - alibi.view(1, H, 1, 1) * (last - pos).clamp(min=0)[:, None].float()
+    if w.sinks is not None:
+        k = torch.cat([k, torch.zeros(S, H, 1, D)], dim=2)
+        v = torch.cat([v, torch.zeros(S, H, 1, D)], dim=2)
+        bias = torch.cat([bias, w.sinks.float().view(1, H, 1, 1).expand(S, H, QL, 1)], dim=3)
+    out = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, scale=w.scale)
+    return out.permute(0, 2, 1, 3)                                           # [S, QL, H, D]
+
+
+@pytest.mark.parametrize("QL", [2, 4, 8])
+@pytest.mark.parametrize("mods", [dict(), dict(alibi=True, window_left=50)])
+@pytest.mark.parametrize("sinks", [False, True])
+def test_multi_token_queries_match_sdpa(oracle, QL, mods, sinks):
+    w = W.make_test_shaped(batch_size=3, nheads=4, nheads_k=2, d=64, seqlen_k=200, varlen=True, has_sinks=sinks,
+                           fp8=False, seed=11)
+    w.context_lens[0] = QL          # the query tokens are the whole context
+    g = torch.Generator().manual_seed(3)
+    query4 = torch.randn(3, QL, 4, 64, generator=g).to(torch.float16)
+    alibi = torch.rand(4, generator=g) * 0.2 if mods.get("alibi") else None
+    wl = mods.get("window_left", -1)
+    got = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, want_f32=True, alibi_slopes=alibi, window_left=wl)[1]
+    want = _reference_multi(w, query4, alibi, wl)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
+    # the last query token is plain decode on the same cache
+    plain = oracle.attention_ref(query4[:, -1].contiguous(), w.key_cache, w.value_cache, w.block_tables,
+                                 w.context_lens, scale=w.scale, block_size=w.block_size, kv_strides=w.kv_strides(),
+                                 num_kv_heads=w.num_kv_heads, sinks=w.sinks, want_f32=True, alibi_slopes=alibi,
+                                 window_left=wl)[1]
+    torch.testing.assert_close(got[:, -1], plain, rtol=1e-6, atol=1e-7)
