@@ -15,6 +15,7 @@ cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTor
              reference) on the same workload on this box's host cores
 configs      the other four configurations, each timed the same way
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
+query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step)
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
              the asynchronous torch.library operators, and a HIP-graph replay of them
 kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
@@ -188,6 +189,30 @@ def _time_score_modifiers(built, steps, torch, W, runner, dev):
                 algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
 
 
+def _time_query_tokens(built, steps, torch, W, runner, dev, query_len=4):
+    """Configuration 1 with several query tokens per sequence (a speculative-decoding
+    verification step): the K/V bytes are read once for all of them."""
+    from flash_attention_factory_amd.lib import paged_attention_loop
+    w, ks, vs = built
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    query4 = torch.randn((S, query_len, H, D), device=dev).to(w.query.dtype)
+    out4 = torch.zeros_like(query4)
+    view = (lambda t: t.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR else (lambda t: t)
+    ts = []
+    for it in range(5 + steps):
+        k = it % len(ks)
+        t = paged_attention_loop.run(None, None, None, out4, None, query4, view(ks[k]), view(vs[k]), w.block_tables,
+                                     w.context_lens, H // Hk, w.scale, B, 0, None, w.sinks, 0.0)
+        if it >= 5:
+            ts.append(t[0])
+    us = float(torch.tensor(ts, dtype=torch.float64).mean())
+    nbytes = w.algorithmic_bytes() + 2 * S * (query_len - 1) * H * D * 2
+    return dict(workload=f"config1 with {query_len} query tokens per sequence, causal (grid-form kernel)",
+                kernel="paged_attn_kernel<128, F16, kv16, loop, extended>", steps=steps, us_per_call=us,
+                algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
+
+
 def _time_stream_ordered(steps, torch, W, runner, dev):
     """Host cost of one small decode step (configuration 0: KV-cache append of one token per
     sequence, then the loop kernel) three ways: the timed `run` calls, which block on every
@@ -306,6 +331,7 @@ def main():
         "configs": others,
     }
     line["score_modifiers"] = _time_score_modifiers(built[1], max(20, args.steps // 2), torch, W, runner, dev)
+    line["query_tokens"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev)
     # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
     e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
     _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)

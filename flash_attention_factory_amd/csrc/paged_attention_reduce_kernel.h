@@ -99,6 +99,9 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   float M = ml0;
   for (int q = 64 + lane; q < np; q += 64) M = fmaxf(M, ml[q * stride]);
   M = wave_max(M);
+  // a row none of whose partitions saw a key (a query token placed before key 0): every
+  // max is -inf and every sum 0; keep exp(m - M) finite so that the row comes out as zeros
+  if (M == -INFINITY) M = 0.f;
 
   float acc[EPL];
 #pragma unroll
@@ -121,7 +124,7 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   }
   W = wave_sum(W);
 
-  const float inv = 1.0f / W;
+  const float inv = W > 0.f ? 1.0f / W : 0.f;
   float o[EPL];
   if constexpr (kReduceWaves == 1) {
 #pragma unroll

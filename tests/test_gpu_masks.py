@@ -155,3 +155,40 @@ def test_query_tokens_with_modifiers_and_last_token_equals_decode(oracle):
         wq.query = query4[:, -1].contiguous().to(_dev())
         single = _call(wq, kernel, **dict(mods))
         torch.testing.assert_close(got[:, -1].float(), single.float(), atol=2e-3, rtol=2e-2)
+
+
+@pytest.mark.parametrize("sinks", [False, True])
+def test_query_block_longer_than_the_context(oracle, sinks):
+    """Leading query tokens that lie before key 0 see nothing: zeros, never NaN."""
+    QL = 4
+    w = W.make_test_shaped(batch_size=3, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True, has_sinks=sinks,
+                           seed=17)
+    w.context_lens[0] = 2
+    w.context_lens[1] = 1
+    g = torch.Generator().manual_seed(8)
+    query4 = torch.randn(3, QL, 8, 128, generator=g).to(torch.float16)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, want_f32=True)[1]
+    assert (ref[0, :2] == 0).all() and (ref[1, :3] == 0).all()
+    wd = w.to(_dev())
+    for kernel in ("loop", "reduce"):
+        got = _call_multi(wd, query4.to(_dev()), kernel).float().cpu()
+        assert (got[0, :2] == 0).all() and (got[1, :3] == 0).all(), kernel
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL)
+
+
+def test_query_tokens_head_major_e4m3(oracle):
+    """The measured pool layout and the second FP8 format with several query tokens."""
+    w = W.make_config(3, num_seqs=4, pool_blocks=400, lens=[1500, 513, 16, 1024], fp8_dtype=torch.float8_e4m3fn)
+    H = w.query.shape[1]
+    QL = 8
+    g = torch.Generator().manual_seed(9)
+    query4 = torch.randn(4, QL, H, 128, generator=g).to(torch.float16)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               fp8_scale=w.fp8_scale, want_f32=True)[1]
+    wd = w.to(_dev())
+    for kernel in ("fp8_loop", "fp8_reduce"):
+        got = _call_multi(wd, query4.to(_dev()), kernel).float().cpu()
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel}: {m}")

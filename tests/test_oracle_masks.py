@@ -114,3 +114,28 @@ def test_multi_token_queries_match_sdpa(oracle, QL, mods, sinks):
                                  num_kv_heads=w.num_kv_heads, sinks=w.sinks, want_f32=True, alibi_slopes=alibi,
                                  window_left=wl)[1]
     torch.testing.assert_close(got[:, -1], plain, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("sinks", [False, True])
+def test_query_tokens_before_the_first_key_see_nothing(oracle, sinks):
+    """A context shorter than the query block: the leading query tokens lie before key 0.  With a
+    sink upstream's formula (test_paged.py:107-121) gives them zeros (all weight on the sink, whose
+    value row is zero); without one it divides 0 by 0 -- the oracle returns zeros there too, which
+    is what attention kernels (SDPA included) store for a row without keys."""
+    QL = 4
+    w = W.make_test_shaped(batch_size=2, nheads=4, nheads_k=2, d=64, seqlen_k=100, varlen=True, has_sinks=sinks,
+                           fp8=False, seed=12)
+    w.context_lens[0] = 2            # tokens 0 and 1 see nothing, token 2 key 0, token 3 keys 0..1
+    g = torch.Generator().manual_seed(5)
+    query4 = torch.randn(2, QL, 4, 64, generator=g).to(torch.float16)
+    got = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, want_f32=True)[1]
+    assert (got[0, :2] == 0).all()
+    want = _reference_multi(w, query4)
+    # this torch's SDPA stores zeros for a row whose keys are all masked, with or without a sink
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
+    if not sinks:
+        # token 2 sees exactly one key: its output is that key's value row
+        v0 = dense_kv(w, w.value_cache)[0, 0]                        # [Hk, D]
+        torch.testing.assert_close(got[0, 2], v0.repeat_interleave(2, dim=0), rtol=1e-6, atol=1e-7)
