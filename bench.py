@@ -16,6 +16,7 @@ cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTor
 configs      the other four configurations, each timed the same way
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
 query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step)
+kv_block_scales  the FP8 loop configuration with E4M3 pools and per-block K and V scales
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
              the asynchronous torch.library operators, and a HIP-graph replay of them
 kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
@@ -213,6 +214,34 @@ def _time_query_tokens(built, steps, torch, W, runner, dev, query_len=4):
                 algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
 
 
+def _time_block_scales(built, steps, torch, W, runner, dev):
+    """The FP8 loop configuration with E4M3 pools and one K and one V scale per physical block
+    and kv head (two more fp32 per 16-token tile of 4 KiB)."""
+    from flash_attention_factory_amd.lib import paged_attention_fp8_loop
+    w, ks, vs = built
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    NB = w.key_cache.shape[0]
+    k_scales = torch.rand((NB, Hk), device=dev) * 0.02 + 0.005
+    v_scales = torch.rand((NB, Hk), device=dev) * 0.02 + 0.005
+    bufs = runner.alloc_buffers(w)
+    view = (lambda t: t.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR else (lambda t: t)
+    ts = []
+    for it in range(5 + steps):
+        k = it % len(ks)
+        t = paged_attention_fp8_loop.run(None, None, None, bufs.out, None, w.query, view(ks[k]), view(vs[k]),
+                                         w.block_tables, w.context_lens, H // Hk, w.scale, 1.0, B, 0, None, w.sinks,
+                                         0.0, k_scales=k_scales, v_scales=v_scales)
+        if it >= 5:
+            ts.append(t[0])
+    us = float(torch.tensor(ts, dtype=torch.float64).mean())
+    blocks = sum(-(-int(c) // B) for c in w.context_lens.tolist())
+    nbytes = w.algorithmic_bytes() + blocks * Hk * 2 * 4
+    return dict(workload="config3 (E4M3 pools) with per-block K and V scales (grid-form kernel)",
+                kernel="paged_attn_kernel<128, F16, e4m3, loop, extended>", steps=steps, us_per_call=us,
+                algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
+
+
 def _time_stream_ordered(steps, torch, W, runner, dev):
     """Host cost of one small decode step (configuration 0: KV-cache append of one token per
     sequence, then the loop kernel) three ways: the timed `run` calls, which block on every
@@ -337,6 +366,7 @@ def main():
     _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
     r["workload"] += "_e4m3"
     others.append(r)
+    line["kv_block_scales"] = _time_block_scales(e4m3, max(20, args.steps // 2), torch, W, runner, dev)
     del e4m3
     line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:

@@ -40,6 +40,10 @@ FA_KV_CACHE_E4M3 = 2
 FA_FP8_E5M2 = 0
 FA_FP8_E4M3 = 1
 
+FA_KV_SCALE_TENSOR = 0
+FA_KV_SCALE_HEAD = 1
+FA_KV_SCALE_BLOCK = 2
+
 FA_MASK_ALIBI = 1
 FA_MASK_SOFTCAP = 2
 FA_MASK_WINDOW = 4
@@ -76,7 +80,9 @@ class Options(ctypes.Structure):
         ("mask_flags", ctypes.c_int32),
         ("window_left", ctypes.c_int32),
         ("query_len", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("kv_scale_mode", ctypes.c_int32),
+        ("k_scales", ctypes.c_void_p),
+        ("v_scales", ctypes.c_void_p),
     ]
 
 
@@ -95,6 +101,29 @@ class KvWriteShape(ctypes.Structure):
         ("cache_dtype", ctypes.c_int32),
         ("num_pool_blocks", ctypes.c_int64),
     ]
+
+
+def set_kv_scales(op: "Options", k_scales, v_scales, num_kv_heads: int, num_pool_blocks: int, device) -> None:
+    """Fill the scale fields of `op` from two fp32 device tensors shaped [num_kv_heads]
+    (per-head scales) or [num_pool_blocks, num_kv_heads] (per-block scales)."""
+    import torch
+    if (k_scales is None) != (v_scales is None):
+        raise PagedAttentionError(FA_ERR_NULL_POINTER, "k_scales and v_scales come together")
+    if k_scales is None:
+        return
+    for t in (k_scales, v_scales):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.device != device or t.shape != k_scales.shape:
+            raise PagedAttentionError(FA_ERR_BAD_SHAPE, "k_scales / v_scales must be contiguous fp32 device tensors of one shape")
+    if tuple(k_scales.shape) == (num_kv_heads,):
+        op.kv_scale_mode = FA_KV_SCALE_HEAD
+    elif tuple(k_scales.shape) == (num_pool_blocks, num_kv_heads):
+        op.kv_scale_mode = FA_KV_SCALE_BLOCK
+    else:
+        raise PagedAttentionError(FA_ERR_BAD_SHAPE,
+                                  f"scales of shape {tuple(k_scales.shape)} are neither [{num_kv_heads}] (per kv head) "
+                                  f"nor [{num_pool_blocks}, {num_kv_heads}] (per block and kv head)")
+    op.k_scales = k_scales.data_ptr()
+    op.v_scales = v_scales.data_ptr()
 
 
 class PagedAttentionError(RuntimeError):

@@ -41,7 +41,15 @@ struct KvWriteParams {
   int64_t kv_head_bytes;
   int64_t src_token_bytes;    // source strides in BYTES
   int64_t src_head_bytes;
+  // SCALED == kWriteScaleArrays: per kv head ([Hk], scale_block_pitch 0) or per destination
+  // block and kv head ([pool blocks, Hk], scale_block_pitch Hk) fp32 scales of K and of V
+  const float *k_scales;
+  const float *v_scales;
+  int32_t scale_block_pitch;
 };
+
+// How the writer scales before rounding: not at all, by one scalar, by scales from arrays.
+constexpr int kWriteUnscaled = 0, kWriteScaleScalar = 1, kWriteScaleArrays = 2;
 
 template <typename ST>
 __device__ __forceinline__ float f32_from_half_of(uint32_t w, int hi) {
@@ -61,7 +69,7 @@ __device__ __forceinline__ float f32_from_half_of(uint32_t w, int hi) {
 // E4M3: v_cvt_pk_fp8_f32 likewise; the format has no infinity and the cast turns everything
 // that rounds beyond 448 (480 and above, NaN included) into NaN, 0x7f | sign, which is
 // decided here from the inputs, whatever the instruction does with them.
-template <typename ST, int KVF, bool SCALED>
+template <typename ST, int KVF, int SCALED>
 __device__ __forceinline__ u32x2 fp8_from_row_piece(u32x4 src, float mul) {
   float f[8];
 #pragma unroll
@@ -69,7 +77,7 @@ __device__ __forceinline__ u32x2 fp8_from_row_piece(u32x4 src, float mul) {
     f[2 * k] = f32_from_half_of<ST>(src[k], 0);
     f[2 * k + 1] = f32_from_half_of<ST>(src[k], 1);
   }
-  if constexpr (SCALED) {
+  if constexpr (SCALED != kWriteUnscaled) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) f[k] *= mul;
   }
@@ -108,7 +116,7 @@ __device__ __forceinline__ u32x2 fp8_from_row_piece(u32x4 src, float mul) {
   return out;
 }
 
-template <typename ST, int KVF, bool SCALED>
+template <typename ST, int KVF, int SCALED>
 __global__ void __launch_bounds__(256) kv_cache_write_kernel(const KvWriteParams p) {
   constexpr bool KV8 = KVF != kKv16;
   const int ppt = p.pieces_per_token;
@@ -136,8 +144,14 @@ __global__ void __launch_bounds__(256) kv_cache_write_kernel(const KvWriteParams
       const uint32_t row = s - block * (uint32_t)p.block_size;
       const int64_t dst = (int64_t)block * p.kv_block_bytes + (int64_t)row * p.kv_token_bytes + dst_off;
       if constexpr (KV8) {
-        *reinterpret_cast<u32x2 *>(p.key_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(k, p.inv_scale);
-        *reinterpret_cast<u32x2 *>(p.value_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(v, p.inv_scale);
+        float k_mul = p.inv_scale, v_mul = p.inv_scale;
+        if constexpr (SCALED == kWriteScaleArrays) {
+          const int64_t at = (int64_t)block * p.scale_block_pitch + head;
+          k_mul = 1.0f / p.k_scales[at];  // correctly rounded, as the host's 1.0f / scale
+          v_mul = 1.0f / p.v_scales[at];
+        }
+        *reinterpret_cast<u32x2 *>(p.key_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(k, k_mul);
+        *reinterpret_cast<u32x2 *>(p.value_cache + dst) = fp8_from_row_piece<ST, KVF, SCALED>(v, v_mul);
       } else {
         *reinterpret_cast<u32x4 *>(p.key_cache + dst) = k;
         *reinterpret_cast<u32x4 *>(p.value_cache + dst) = v;

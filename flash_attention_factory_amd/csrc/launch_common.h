@@ -60,6 +60,9 @@ struct Resolved {
   float softcap;
   int32_t window_left;
   int32_t query_len;  // query tokens per sequence, >= 1
+  int32_t kv_scale_mode;  // fa_kv_scale; with a mode other than 0 fp8_scale is 1
+  const float *k_scales;
+  const float *v_scales;
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -151,6 +154,21 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->softcap = o ? o->softcap : 0.f;
   r->window_left = o ? o->window_left : 0;
   r->fp8_scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
+  r->kv_scale_mode = (kv8 && o) ? o->kv_scale_mode : FA_KV_SCALE_TENSOR;
+  r->k_scales = r->v_scales = nullptr;
+  if (r->kv_scale_mode != FA_KV_SCALE_TENSOR) {
+    if (r->kv_scale_mode != FA_KV_SCALE_HEAD && r->kv_scale_mode != FA_KV_SCALE_BLOCK)
+      return fail(FA_ERR_BAD_SHAPE, "kv_scale_mode %d is none of tensor (0), head (1), block (2)", r->kv_scale_mode);
+    if (!o->k_scales || !o->v_scales)
+      return fail(FA_ERR_NULL_POINTER, "kv_scale_mode %d needs k_scales and v_scales", r->kv_scale_mode);
+    if (((uintptr_t)o->k_scales | (uintptr_t)o->v_scales) % 4)
+      return fail(FA_ERR_BAD_SHAPE, "k_scales and v_scales must be 4-byte aligned");
+    if (r->kv_scale_mode == FA_KV_SCALE_BLOCK && s->num_pool_blocks <= 0)
+      return fail(FA_ERR_BAD_SHAPE, "per-block scales need num_pool_blocks");
+    r->k_scales = o->k_scales;
+    r->v_scales = o->v_scales;
+    r->fp8_scale = 1.0f;
+  }
   r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   r->elapsed_us = o ? o->elapsed_us : nullptr;
   r->validate_only = o && o->validate_only != 0;
@@ -180,6 +198,9 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.window_left = r.window_left;
   p.query_len = r.query_len;
   p.out_scale = r.fp8_scale;
+  p.kv_scale_mode = r.kv_scale_mode;
+  p.k_scales = r.k_scales;
+  p.v_scales = r.v_scales;
   p.num_seqs = s.num_seqs;
   p.num_heads = s.num_heads;
   p.num_kv_heads = s.num_kv_heads;

@@ -28,24 +28,28 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
   const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
-  if (r.mask_flags != 0 || r.query_len > 1) {
-    // score modifiers, several query tokens: the grid form has the instance for them
+  // score modifiers, several query tokens, per-head or per-block scales: the extended instances
+  const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
+  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
+      max_ctx < kLoopPersistentMaxContext) {
+    // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
+    // sequences first, with the next item's first loads issued before each merge.
+    constexpr int PW = PersistentLoop<KV8>::waves;
+    auto plain = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                   Pipeline<KV8>::tiles_per_chunk, false>;
+    auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                      Pipeline<KV8>::tiles_per_chunk, true>;
+    auto kernel = ext ? extended : plain;
+    int resident = 0;
+    FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
+    const dim3 grid((unsigned)std::min<int64_t>(resident, items));
+    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
+  } else if (ext) {
     const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(
         paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
                           Pipeline<KV8>::tiles_per_chunk, true>,
         grid, dim3(NW * 64), 0, p));
-  } else if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
-             max_ctx < kLoopPersistentMaxContext) {
-    // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
-    // sequences first, with the next item's first loads issued before each merge.
-    constexpr int PW = PersistentLoop<KV8>::waves;
-    auto kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                    Pipeline<KV8>::tiles_per_chunk>;
-    int resident = 0;
-    FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
-    const dim3 grid((unsigned)std::min<int64_t>(resident, items));
-    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
   } else {
     const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(

@@ -32,25 +32,29 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // work-group per (kv head, partition slot, sequence); slots past a sequence's length
   // return at once and write nothing (paged_attention_kernel_v2.hpp:577-579).
   int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
-  if (r.mask_flags != 0 || r.query_len > 1) {
-    // score modifiers, several query tokens: the grid form has the instance for them
-    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
-    FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
-                          Pipeline<KV8>::tiles_per_chunk, true>,
-        grid, dim3(NW * 64), 0, p));
-  } else if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
+  // score modifiers, several query tokens, per-head or per-block scales: the extended instances
+  const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
+  if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
       (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
     // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
     constexpr int SW = SegmentSplit<KV8>::waves;
-    auto kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                            Pipeline<KV8>::tiles_per_chunk>;
+    auto plain = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                           Pipeline<KV8>::tiles_per_chunk, false>;
+    auto extended = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                              Pipeline<KV8>::tiles_per_chunk, true>;
+    auto kernel = ext ? extended : plain;
     int resident = 0;
     FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
     const int64_t max_items =
         (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
     segment_groups = (int)std::min<int64_t>(resident, max_items);
     FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
+  } else if (ext) {
+    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+    FA_HIP_CHECK(timer.launch(
+        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
+                          Pipeline<KV8>::tiles_per_chunk, true>,
+        grid, dim3(NW * 64), 0, p));
   } else {
     const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
     FA_HIP_CHECK(timer.launch(

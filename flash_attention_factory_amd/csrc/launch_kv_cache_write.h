@@ -45,6 +45,15 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   if (((uintptr_t)key | (uintptr_t)value | (uintptr_t)key_cache | (uintptr_t)value_cache) % 16 ||
       (uintptr_t)slot_mapping % 8)
     return fail(FA_ERR_BAD_SHAPE, "key, value and the pools must be 16-byte aligned, slot_mapping 8-byte aligned");
+  const int scale_mode = (kv8 && o) ? o->kv_scale_mode : FA_KV_SCALE_TENSOR;
+  if (scale_mode != FA_KV_SCALE_TENSOR) {
+    if (scale_mode != FA_KV_SCALE_HEAD && scale_mode != FA_KV_SCALE_BLOCK)
+      return fail(FA_ERR_BAD_SHAPE, "kv_scale_mode %d is none of tensor (0), head (1), block (2)", scale_mode);
+    if (!o->k_scales || !o->v_scales)
+      return fail(FA_ERR_NULL_POINTER, "kv_scale_mode %d needs k_scales and v_scales", scale_mode);
+    if (((uintptr_t)o->k_scales | (uintptr_t)o->v_scales) % 4)
+      return fail(FA_ERR_BAD_SHAPE, "k_scales and v_scales must be 4-byte aligned");
+  }
   if (o && o->validate_only) return FA_OK;
   if (s->num_tokens == 0) {
     if (o && o->elapsed_us) o->elapsed_us[0] = 0.f;
@@ -63,7 +72,7 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   p.key_cache = reinterpret_cast<char *>(key_cache);
   p.value_cache = reinterpret_cast<char *>(value_cache);
   p.slot_mapping = slot_mapping;
-  const float scale = (kv8 && o && o->fp8_scale != 0.f) ? o->fp8_scale : 1.0f;
+  const float scale = (kv8 && o && o->fp8_scale != 0.f && scale_mode == FA_KV_SCALE_TENSOR) ? o->fp8_scale : 1.0f;
   p.inv_scale = 1.0f / scale;
   p.num_tokens = s->num_tokens;
   p.pieces_per_row = s->head_size / 8;
@@ -77,6 +86,9 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   p.kv_head_bytes = s->kv_head_stride * eb;
   p.src_token_bytes = src_token * 2;
   p.src_head_bytes = src_head * 2;
+  p.k_scales = scale_mode != FA_KV_SCALE_TENSOR ? o->k_scales : nullptr;
+  p.v_scales = scale_mode != FA_KV_SCALE_TENSOR ? o->v_scales : nullptr;
+  p.scale_block_pitch = scale_mode == FA_KV_SCALE_BLOCK ? s->num_kv_heads : 0;
 
   hipStream_t stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   KernelTimer timer(o && o->elapsed_us, stream);
@@ -84,17 +96,24 @@ inline fa_status launch_kv_cache_write(const void *key, const void *value, void 
   const int64_t groups_needed = ((int64_t)s->num_tokens + p.tokens_per_group - 1) / p.tokens_per_group;
   const dim3 grid((unsigned)std::min<int64_t>(groups_needed, 0x7fffffff)), block(256);
   const bool bf16 = s->src_dtype == FA_DTYPE_BF16;
-  const bool scaled = scale != 1.0f;
+  const int scaled = scale_mode != FA_KV_SCALE_TENSOR ? kWriteScaleArrays
+                     : scale != 1.0f                   ? kWriteScaleScalar
+                                                       : kWriteUnscaled;
 #define FA_KVW_LAUNCH(ST, KVF, SC) FA_HIP_CHECK(timer.launch(kv_cache_write_kernel<ST, KVF, SC>, grid, block, 0, p))
+#define FA_KVW_SCALED(ST, KVF)                                             \
+  do {                                                                     \
+    if (scaled == kWriteScaleArrays) FA_KVW_LAUNCH(ST, KVF, kWriteScaleArrays);       \
+    else if (scaled == kWriteScaleScalar) FA_KVW_LAUNCH(ST, KVF, kWriteScaleScalar);  \
+    else FA_KVW_LAUNCH(ST, KVF, kWriteUnscaled);                           \
+  } while (0)
   if (!kv8) {  // a 16-bit pool takes bit copies whatever the 16-bit type
-    FA_KVW_LAUNCH(F16, kKv16, false);
+    FA_KVW_LAUNCH(F16, kKv16, kWriteUnscaled);
   } else if (e4m3) {
-    if (bf16) { if (scaled) FA_KVW_LAUNCH(BF16, kKvE4M3, true); else FA_KVW_LAUNCH(BF16, kKvE4M3, false); }
-    else { if (scaled) FA_KVW_LAUNCH(F16, kKvE4M3, true); else FA_KVW_LAUNCH(F16, kKvE4M3, false); }
+    if (bf16) FA_KVW_SCALED(BF16, kKvE4M3); else FA_KVW_SCALED(F16, kKvE4M3);
   } else {
-    if (bf16) { if (scaled) FA_KVW_LAUNCH(BF16, kKvE5M2, true); else FA_KVW_LAUNCH(BF16, kKvE5M2, false); }
-    else { if (scaled) FA_KVW_LAUNCH(F16, kKvE5M2, true); else FA_KVW_LAUNCH(F16, kKvE5M2, false); }
+    if (bf16) FA_KVW_SCALED(BF16, kKvE5M2); else FA_KVW_SCALED(F16, kKvE5M2);
   }
+#undef FA_KVW_SCALED
 #undef FA_KVW_LAUNCH
   if (o && o->elapsed_us) FA_HIP_CHECK(timer.read(0, &o->elapsed_us[0]));
   return FA_OK;

@@ -72,7 +72,9 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   }
 
   if (!wa.col_valid) return;
-  const float inv = L > 0.f ? p.out_scale / L : 0.f;  // L = 0: nothing visible (local window, causal rule)
+  float out_scale = p.out_scale;
+  if constexpr (W::kExt) out_scale = wa.out_mul;
+  const float inv = L > 0.f ? out_scale / L : 0.f;  // L = 0: nothing visible (local window, causal rule)
   const int head = kvh * p.group + wa.col_g;
   const int64_t row = W::kExt ? (int64_t)seq * p.query_len + wa.col_q : seq;  // row of query / out / scratch
   const int d0 = 4 * r * NDT + wave * SL;  // first head-dim element this lane stores
@@ -131,11 +133,11 @@ paged_attn_kernel(const PagedAttnParams p) {
   wa.load_q(seq, kvh);
   wa.reset(wa.load_sink(kvh, wave == 0 && (!PART || part == 0)));
   int c_lo = c_begin;  // first chunk that holds a visible token
+  typename W::ItemExt ext = {};
   if constexpr (MASKS) {
-    wa.load_slope(kvh);
-    wa.set_context(ctx);
-    // the earliest query token's window decides where reading starts
-    if (p.mask_flags & kMaskWindow) c_lo = max(c_begin, max(0, ctx - p.query_len - p.window_left) / CT);
+    ext = wa.fetch_item_ext(kvh, table);
+    wa.set_item(ext, ctx);
+    c_lo = wa.first_visible_chunk(ctx, c_begin);  // the earliest query token's window decides
   }
 
   // ---- streaming loop ------------------------------------------------------------------
@@ -153,19 +155,23 @@ paged_attn_kernel(const PagedAttnParams p) {
     Chunk R;
     wa.issue_k(R, kvh, ci, ids0);
     wa.issue_v(R, kvh, ci, ids0);
+    typename W::TileScales ts = {}, nts = {};  // extended instances only
+    if constexpr (MASKS) ts = wa.fetch_scales(ids0, kvh, ext);
     Ids nids = wa.fetch_ids(table, ci + NW, last_blk);
     while (ci + NW < c_end) {
       const int cn = ci + NW;
       const auto s = wa.qk(R);
       wa.issue_k(R, kvh, cn, nids);
-      const auto pb = wa.template soft<false, MASKS>(R, s, ci, tok_end);
+      if constexpr (MASKS) nts = wa.fetch_scales(nids, kvh, ext);
+      const auto pb = wa.template soft<false, MASKS>(R, s, ci, tok_end, &ts);
       wa.pv(R, pb);
       wa.issue_v(R, kvh, cn, nids);
       nids = wa.fetch_ids(table, cn + NW, last_blk);
+      ts = nts;
       ci = cn;
     }
     const auto s = wa.qk(R);
-    wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end));
+    wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end, &ts));
   }
 
   merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part);

@@ -15,6 +15,11 @@
 //     wavefronts have as a rule long delivered theirs: there is no barrier between items
 //     and the stream never drains.
 // Built for up to 128 sequences of fewer than 2^24 tokens; anything else uses the grid form.
+//
+// EXT: the extended instance (score modifiers, several query tokens per sequence, per-head or
+// per-block FP8 scales; see WaveAttn).  An item then also brings its ALiBi slope and scales,
+// requested one item ahead like the query rows; chunks wholly before a local window are
+// skipped, so an item starts at its first visible chunk.
 #pragma once
 
 #include "paged_attention_kernel.h"
@@ -28,12 +33,14 @@ constexpr int kLoopPersistentMaxContext = 1 << 24;  // lengths are packed into 2
 // item -- it only turns a would-be hang into a wrong answer that the tests catch.
 constexpr int kLoopPersistentSpinLimit = 1 << 24;
 
-template <int D, typename QT, int KVF, int NW, int OCC, int TPC>
+template <int D, typename QT, int KVF, int NW, int OCC, int TPC, bool EXT = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KVF, TPC, Pipeline<(KVF != 0)>::stream_loads_loop>;
+  using W = WaveAttn<D, QT, KVF, TPC, Pipeline<(KVF != 0)>::stream_loads_loop, EXT>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
+  using ItemExt = typename W::ItemExt;
+  using TileScales = typename W::TileScales;
   constexpr int CT = W::CT;
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
@@ -90,7 +97,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       rank1 += ku > key1;
     }
   }
-  struct Item { int seq, kvh, ctx, c_end; };
+  struct Item { int seq, kvh, ctx, c_end, c_lo; };  // c_lo: first chunk to read (0 unless EXT)
   // n-th item of this work-group: position n*G + j on even n, n*G + G-1-j on odd n
   auto item_at = [&](int n, Item &it) -> bool {
     const int pos = n * G + ((n & 1) ? G - 1 - wg : wg);
@@ -103,6 +110,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     it.seq = __builtin_amdgcn_readfirstlane(s);
     it.ctx = s < 64 ? __builtin_amdgcn_readlane(len0, s) : __builtin_amdgcn_readlane(len1, s - 64);
     it.c_end = (it.ctx + CT - 1) / CT;
+    it.c_lo = 0;
     return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
   };
 
@@ -119,6 +127,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   int n = 0;
   Item cur;
   if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
+  if constexpr (EXT) cur.c_lo = wa.first_visible_chunk(cur.ctx, 0);
   if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
@@ -143,7 +152,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   // wavefront calls finish(item) before it publishes item + 1, and finish(item) returns
   // only after all have published `item`, hence after all have finished item - 1: a
   // buffer is never overwritten while somebody still reads it.
-  auto finish = [&](int item, int seq, int kvh) {
+  auto finish = [&](int item, int seq, int kvh, float out_mul) {
     const int b = item & 1;
     const int target = NW * ((item >> 1) + 1);
     for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
@@ -171,17 +180,24 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + k][lane];
       o[k] = a;
     }
-    if (i < p.group) {
-      const int head = kvh * p.group + i;
+    if (wa.col_valid) {
+      const int head = kvh * p.group + wa.col_g;
       const int d0 = 4 * r * NDT + wave * SL;
-      W::template store_q<SL>(reinterpret_cast<char *>(p.out) +
-                                  (((int64_t)seq * p.num_heads + head) * D + d0) * 2,
-                              o, p.out_scale / L);
+      int64_t row = seq;
+      float inv = p.out_scale / L;
+      if constexpr (EXT) {
+        row = (int64_t)seq * p.query_len + wa.col_q;
+        inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key
+      }
+      W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
     }
   };
 
   // first chunk of the first item
-  bool armed = wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  bool armed = cur.c_lo + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  ItemExt cur_ext = {}, nxt_ext = {};         // extended instances only
+  TileScales ts = {}, nts = {}, nxt_ts = {};
+  if constexpr (EXT) cur_ext = wa.fetch_item_ext(cur.kvh, p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq);
   if (armed) {
     Ids ids;
 #pragma unroll
@@ -190,51 +206,68 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
                                    : __builtin_amdgcn_readlane(sid1[t], cur.seq - 64);
       ids.v[t] = min((uint32_t)raw, (uint32_t)p.max_block_id);
     }
+    if constexpr (EXT) {
+      if (cur.c_lo != 0)  // the ids requested with the lengths are those of chunk `wave`
+        ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_lo + wave, col_max);
+    }
     wa.load_q(cur.seq, cur.kvh);
-    wa.issue_k(R, cur.kvh, wave, ids);
-    wa.issue_v(R, cur.kvh, wave, ids);
+    wa.issue_k(R, cur.kvh, cur.c_lo + wave, ids);
+    wa.issue_v(R, cur.kvh, cur.c_lo + wave, ids);
+    if constexpr (EXT) ts = wa.fetch_scales(ids, cur.kvh, cur_ext);
   }
   uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
+  float prev_out_mul = 1.f;
 
   while (true) {
     Item nxt;
     const bool has_next = item_at(n + 1, nxt);
-    const bool next_armed = has_next && wave < nxt.c_end;
+    if constexpr (EXT) {
+      if (has_next) {
+        nxt.c_lo = wa.first_visible_chunk(nxt.ctx, 0);
+        nxt_ext = wa.fetch_item_ext(nxt.kvh, p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq);
+      }
+    }
+    const bool next_armed = has_next && nxt.c_lo + wave < nxt.c_end;
     Ids nxt_ids = {};
     if (next_armed)
-      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, wave, col_max);
+      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_lo + wave, col_max);
 
     wa.reset(sink_raw);
+    if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
     uint32_t next_sink = W::kNoSink;
     bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;
-      int ci = wave;
+      int ci = cur.c_lo + wave;
       Ids nids = wa.fetch_ids(table, ci + NW, col_max);
       if (ci + NW < cur.c_end) {
         {  // first chunk of the item, then the merge owed to the previous item
           const int cn = ci + NW;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
-          const auto pb = wa.template soft<false>(R, s, ci, cur.ctx);
+          if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
+          const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.ctx, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
           nids = wa.fetch_ids(table, cn + NW, col_max);
+          ts = nts;
           ci = cn;
         }
         if (owed) {
-          finish(n - 1, prev.seq, prev.kvh);
+          finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
           owed = false;
         }
         while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
           const int cn = ci + NW;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
-          const auto pb = wa.template soft<false>(R, s, ci, cur.ctx);
+          if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
+          const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.ctx, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
           nids = wa.fetch_ids(table, cn + NW, col_max);
+          ts = nts;
           ci = cn;
         }
       }
@@ -243,18 +276,20 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       if (next_armed) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
         next_sink = wa.load_sink(nxt.kvh, wave == 0);
-        wa.issue_k(R, nxt.kvh, wave, nxt_ids);
+        wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+        if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
       }
-      const auto pb = wa.template soft<true>(R, s, ci, cur.ctx);
+      const auto pb = wa.template soft<true, EXT>(R, s, ci, cur.ctx, &ts);
       wa.pv(R, pb);
-      if (next_armed) wa.issue_v(R, nxt.kvh, wave, nxt_ids);
+      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
       wa.load_q(nxt.seq, nxt.kvh);
       next_sink = wa.load_sink(nxt.kvh, wave == 0);
-      wa.issue_k(R, nxt.kvh, wave, nxt_ids);
-      wa.issue_v(R, nxt.kvh, wave, nxt_ids);
+      wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
-    if (owed) finish(n - 1, prev.seq, prev.kvh);
+    if (owed) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
     publish(n);
 
     if (!has_next) break;
@@ -262,9 +297,14 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     cur = nxt;
     armed = next_armed;
     sink_raw = next_sink;
+    if constexpr (EXT) {
+      prev_out_mul = cur_ext.out_mul;
+      cur_ext = nxt_ext;
+      ts = nxt_ts;
+    }
     ++n;
   }
-  finish(n, cur.seq, cur.kvh);
+  finish(n, cur.seq, cur.kvh, EXT ? cur_ext.out_mul : 1.f);
 }
 
 }  // namespace fa

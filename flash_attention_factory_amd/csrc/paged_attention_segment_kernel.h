@@ -18,6 +18,12 @@
 // finely, in a batch with a thousand (sequence, kv head) pairs most sequences stay whole.
 // Segments are dealt to the work-groups longest first in snake order (see below).
 // Built for up to 256 sequences; larger batches use the grid form.
+//
+// EXT: the extended instance (score modifiers, several query tokens per sequence, per-head or
+// per-block FP8 scales; see WaveAttn).  Rows of the scratch arrays are then (sequence, query
+// token) pairs.  A segment starts at its first chunk inside the local window; one that lies
+// wholly before the window publishes empty states and stores an empty partial (max -inf,
+// sum 0, zeros), which the reduce kernel weighs with 0.
 #pragma once
 
 #include "paged_attention_kernel.h"
@@ -26,12 +32,14 @@
 
 namespace fa {
 
-template <int D, typename QT, int KVF, int NW, int OCC, int TPC>
+template <int D, typename QT, int KVF, int NW, int OCC, int TPC, bool EXT = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_segment_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KVF, TPC, SegmentSplit<(KVF != 0)>::stream_loads>;
+  using W = WaveAttn<D, QT, KVF, TPC, SegmentSplit<(KVF != 0)>::stream_loads, EXT>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
+  using ItemExt = typename W::ItemExt;
+  using TileScales = typename W::TileScales;
   constexpr int CT = W::CT;
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
@@ -96,7 +104,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     }
   }
 
-  struct Item { int seq, kvh, part0, tok_end, c_begin, c_end; };
+  struct Item { int seq, kvh, part0, tok_end, c_begin, c_end, ctx; };  // ctx: the sequence's length (EXT)
   // position in the sorted list -> (sequence, segment, kv head), kv head fastest
   auto decode = [&](int pos) -> Item {
     Item it;
@@ -133,6 +141,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     it.tok_end = full ? tok_begin + seg_tokens : ctx_s;
     it.c_begin = tok_begin / CT;
     it.c_end = (it.tok_end + CT - 1) / CT;
+    it.ctx = ctx_s;
     return it;
   };
   // n-th item of this work-group
@@ -151,6 +160,10 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   W wa(p, lane);
   const int r = wa.r, i = wa.i;
   Chunk R;
+  // EXT: a segment is read from its first chunk inside the local window
+  auto clip = [&](Item &it) {
+    if constexpr (EXT) it.c_begin = wa.first_visible_chunk(it.ctx, it.c_begin);
+  };
 
   auto publish = [&](int n) {
     const int b = n & 1;
@@ -168,7 +181,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   // Merge the NW published states of the work-group's n-th item, normalise, store this
   // wavefront's slice of the partial (see the persistent loop kernel for why the wait
   // always ends and why a buffer is never overwritten while it is read).
-  auto finish = [&](int n, const Item &it) {
+  auto finish = [&](int n, const Item &it, float out_mul) {
     const int b = n & 1;
     const int target = NW * ((n >> 1) + 1);
     for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
@@ -196,11 +209,17 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + e][lane];
       o[e] = a;
     }
-    if (i < p.group) {
-      const int head = it.kvh * p.group + i;
-      const int64_t slot = ((int64_t)it.seq * p.num_heads + head) * p.max_num_partitions + it.part0;
+    if (wa.col_valid) {
+      const int head = it.kvh * p.group + wa.col_g;
+      int64_t row = it.seq;
+      float inv = p.out_scale / L;
+      if constexpr (EXT) {
+        row = (int64_t)it.seq * p.query_len + wa.col_q;
+        inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key of the segment
+      }
+      const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
       const int d0 = 4 * r * NDT + wave * SL;
-      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, p.out_scale / L);
+      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
       if (r == 0 && wave == 0) {
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;
@@ -210,28 +229,40 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
 
   int n = 0;
   Item cur = decode(position(0));
+  clip(cur);
   // first chunk of the first item
   bool armed = cur.c_begin + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  ItemExt cur_ext = {}, nxt_ext = {};            // extended instances only
+  TileScales ts = {}, nts = {}, nxt_ts = {};
+  if constexpr (EXT) cur_ext = wa.fetch_item_ext(cur.kvh, p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq);
   if (armed) {
     const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_begin + wave, col_max);
     wa.load_q(cur.seq, cur.kvh);
     wa.issue_k(R, cur.kvh, cur.c_begin + wave, ids);
     wa.issue_v(R, cur.kvh, cur.c_begin + wave, ids);
+    if constexpr (EXT) ts = wa.fetch_scales(ids, cur.kvh, cur_ext);
   }
   uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
+  float prev_out_mul = 1.f;
 
   while (true) {
     const int pn = position(n + 1);
     const bool has_next = pn < total_items;
     Item nxt = cur;
-    if (has_next) nxt = decode(pn);
+    if (has_next) {
+      nxt = decode(pn);
+      clip(nxt);
+      if constexpr (EXT)
+        nxt_ext = wa.fetch_item_ext(nxt.kvh, p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq);
+    }
     const bool next_armed = has_next && nxt.c_begin + wave < nxt.c_end;
     Ids nxt_ids = {};
     if (next_armed)
       nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_begin + wave, col_max);
 
     wa.reset(sink_raw);
+    if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
     uint32_t next_sink = W::kNoSink;
     bool owed = n > 0;
     if (armed) {
@@ -243,24 +274,28 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
           const int cn = ci + NW;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
-          const auto pb = wa.template soft<false>(R, s, ci, cur.tok_end);
+          if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
+          const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
           nids = wa.fetch_ids(table, cn + NW, col_max);
+          ts = nts;
           ci = cn;
         }
         if (owed) {
-          finish(n - 1, prev);
+          finish(n - 1, prev, prev_out_mul);
           owed = false;
         }
         while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
           const int cn = ci + NW;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
-          const auto pb = wa.template soft<false>(R, s, ci, cur.tok_end);
+          if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
+          const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
           nids = wa.fetch_ids(table, cn + NW, col_max);
+          ts = nts;
           ci = cn;
         }
       }
@@ -270,8 +305,9 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
         next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
         wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+        if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
       }
-      const auto pb = wa.template soft<true>(R, s, ci, cur.tok_end);
+      const auto pb = wa.template soft<true, EXT>(R, s, ci, cur.tok_end, &ts);
       wa.pv(R, pb);
       if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
@@ -279,8 +315,9 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
       wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
       wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+      if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
-    if (owed) finish(n - 1, prev);
+    if (owed) finish(n - 1, prev, prev_out_mul);
     publish(n);
 
     if (!has_next) break;
@@ -288,9 +325,14 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     cur = nxt;
     armed = next_armed;
     sink_raw = next_sink;
+    if constexpr (EXT) {
+      prev_out_mul = cur_ext.out_mul;
+      cur_ext = nxt_ext;
+      ts = nxt_ts;
+    }
     ++n;
   }
-  finish(n, cur);
+  finish(n, cur, EXT ? cur_ext.out_mul : 1.f);
 }
 
 }  // namespace fa

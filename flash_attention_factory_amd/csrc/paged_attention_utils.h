@@ -173,6 +173,11 @@ __device__ __forceinline__ int32_t load_uniform_i32(const int32_t *p) {
   return *(const_ptr)(uintptr_t)p;
 }
 
+__device__ __forceinline__ float load_uniform_f32(const float *p) {
+  typedef const float __attribute__((address_space(4))) *const_ptr;
+  return *(const_ptr)(uintptr_t)p;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // K/V bytes are read exactly once per launch.  STREAM marks a load non-temporal so that it

@@ -55,9 +55,15 @@ struct PagedAttnParams {
   int32_t window_left;
   int32_t mask_flags;           // kMaskAlibi | kMaskSoftcap | kMaskWindow
   int32_t query_len;            // query tokens per sequence (1 = plain decode)
+  // finer dequantisation scales of an FP8 cache, read only by the extended instances.  With a
+  // mode other than kScaleTensor score_scale is the bare softmax scale and out_scale is 1.
+  int32_t kv_scale_mode;        // kScaleTensor / kScaleHead / kScaleBlock
+  const float *k_scales;        // [Hk] or [pool blocks, Hk] fp32
+  const float *v_scales;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
+constexpr int kScaleTensor = 0, kScaleHead = 1, kScaleBlock = 2;  // = fa_kv_scale of the C ABI
 
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
@@ -88,6 +94,10 @@ struct WaveAttn {
   };
   struct Ids { int v[TPC]; };      // physical block id of every tile of a chunk
   struct Scores { f32x4 v[TPC]; };
+  // EXT, per-block scales: what the scores of each tile are multiplied with (softmax scale x
+  // the tile's K scale) and what its probabilities are multiplied with before P.V (the tile's
+  // V scale over the item's reference V scale)
+  struct TileScales { float k[TPC], v[TPC]; };
   struct Probs { u32x4 v[NP2]; };
 
   const PagedAttnParams &p;
@@ -107,6 +117,8 @@ struct WaveAttn {
   float m, l;
   f32x4 acc[NDT];
   float slope_log2 = 0.f;  // ALiBi slope of head i in base-2 units (MASKS instances only)
+  // EXT: what the normalised output of the item at hand is multiplied with (see ItemExt).
+  float out_mul = 1.f;
 
   __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
       : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {
@@ -120,13 +132,71 @@ struct WaveAttn {
     }
   }
 
-  // EXT: the context length of the item at hand; query token q sits at position
-  // ctx - query_len + q and sees the keys up to there.
-  __device__ __forceinline__ void set_context(int ctx) { col_last = ctx - p.query_len + col_q; }
+  // EXT: what an item (sequence, kv head) brings besides its query rows.  fetch_item_ext only
+  // requests the values, so that a persistent kernel can ask for the next item's while the
+  // current one still streams; set_item makes them the ones soft() works with.
+  struct ItemExt {
+    float slope_log2;  // ALiBi slope of this lane's head, base-2 units
+    float k_mul;       // raw score -> scaled score: softmax scale x K scale (tensor or head)
+    float out_mul;     // what the normalised output is multiplied with: V scale (tensor or
+                       // head), or with per-block scales the item's reference V scale
+    float inv_v_ref;   // per-block scales: 1 / out_mul
+  };
 
-  // ALiBi slope of this lane's head; kernels built with MASKS call it once per item.
-  __device__ __forceinline__ void load_slope(int kvh) {
-    slope_log2 = ((p.mask_flags & kMaskAlibi) && col_valid) ? p.alibi_slopes[kvh * p.group + col_g] * kLog2e : 0.f;
+  // `table`: the sequence's row of the block table; its first block's V scale serves as the
+  // item's reference with per-block scales.
+  __device__ __forceinline__ ItemExt fetch_item_ext(int kvh, const int32_t *table) const {
+    ItemExt x;
+    x.slope_log2 =
+        ((p.mask_flags & kMaskAlibi) && col_valid) ? p.alibi_slopes[kvh * p.group + col_g] * kLog2e : 0.f;
+    x.k_mul = p.score_scale;
+    x.out_mul = p.out_scale;
+    x.inv_v_ref = 1.f;
+    if constexpr (KV8) {
+      if (p.kv_scale_mode == kScaleHead) {
+        x.k_mul = p.score_scale * load_uniform_f32(p.k_scales + kvh);
+        x.out_mul = load_uniform_f32(p.v_scales + kvh);
+      } else if (p.kv_scale_mode == kScaleBlock) {
+        const uint32_t b0 = min((uint32_t)load_uniform_i32(table), (uint32_t)p.max_block_id);
+        x.out_mul = load_uniform_f32(p.v_scales + (int64_t)b0 * p.num_kv_heads + kvh);
+        x.inv_v_ref = 1.0f / x.out_mul;
+      }
+    }
+    return x;
+  }
+
+  // Query token q of the item sits at position ctx - query_len + q and sees the keys up to there.
+  __device__ __forceinline__ void set_item(const ItemExt &x, int ctx) {
+    slope_log2 = x.slope_log2;
+    out_mul = x.out_mul;
+    col_last = ctx - p.query_len + col_q;
+  }
+
+  // First chunk that holds a key some query token of the item sees (local window), at least c_begin.
+  __device__ __forceinline__ int first_visible_chunk(int ctx, int c_begin) const {
+    if (!(p.mask_flags & kMaskWindow)) return c_begin;
+    return max(c_begin, max(0, ctx - p.query_len - p.window_left) / CT);
+  }
+
+  // EXT: multipliers of a chunk's tiles (uniform over the item unless the scales are per block).
+  __device__ __forceinline__ TileScales fetch_scales(const Ids &ids, int kvh, const ItemExt &x) const {
+    TileScales ts;
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) {
+      ts.k[t] = x.k_mul;
+      ts.v[t] = 1.0f;
+    }
+    if constexpr (KV8) {
+      if (p.kv_scale_mode == kScaleBlock) {
+#pragma unroll
+        for (int t = 0; t < TPC; ++t) {
+          const int64_t at = (int64_t)ids.v[t] * p.num_kv_heads + kvh;
+          ts.k[t] = p.score_scale * load_uniform_f32(p.k_scales + at);
+          ts.v[t] = load_uniform_f32(p.v_scales + at) * x.inv_v_ref;
+        }
+      }
+    }
+    return ts;
   }
 
   __device__ __forceinline__ void load_q(int seq, int kvh) {
@@ -261,7 +331,8 @@ struct WaveAttn {
   // window, ALiBi, in that order (upstream test_paged.py:92-110) -- and the causal rule, all
   // relative to the position col_last of this column's query token.
   template <bool CHECK_TAIL, bool MASKS = false>
-  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end) {
+  __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end,
+                                        const TileScales *ts = nullptr) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
     float t[NT];
     if constexpr (MASKS) {
@@ -270,7 +341,7 @@ struct WaveAttn {
       const int first_visible = (p.mask_flags & kMaskWindow) ? col_last - p.window_left : 0;
 #pragma unroll
       for (int e = 0; e < NT; ++e) {
-        float x = s.v[e >> 2][e & 3] * p.score_scale;
+        float x = s.v[e >> 2][e & 3] * ts->k[e >> 2];
         if (cap) {  // cap * tanh(x / cap), tanh(z) = 1 - 2 / (exp(2z) + 1)
           const float e2 = fast_exp2(x * inv_cap2);
           x = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f));
@@ -320,6 +391,10 @@ struct WaveAttn {
     }
     // k-slots (r, e) of step pr = this lane's eight tokens of the step, rounded to the q
     // dtype (paged_attention_kernel_loop.hpp:404-407)
+    if constexpr (MASKS && KV8) {  // per-block V scales ride on the probabilities (1.0 otherwise)
+#pragma unroll
+      for (int e = 0; e < NT; ++e) t[e] *= ts->v[e >> 2];
+    }
     Probs pb;
 #pragma unroll
     for (int pr = 0; pr < NP2; ++pr)

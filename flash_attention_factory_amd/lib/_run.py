@@ -42,7 +42,8 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
              num_queries_per_tokens: int, sm_scale: float, fp8_scale: float, block_size: int,
              max_context_len: int, alibi_slopes, sinks: Optional[torch.Tensor], softcap: float,
              partition_size: int = 0, timed: bool = True, apply_alibi: bool = False,
-             apply_softcap: bool = False, window_left: Optional[int] = None) -> List[float]:
+             apply_softcap: bool = False, window_left: Optional[int] = None,
+             k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None) -> List[float]:
     L = _cabi.load()
     if not query.is_cuda:
         raise RuntimeError("paged attention runs on the GPU only: `query` is not a device tensor")
@@ -106,6 +107,10 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
         op.mask_flags |= _cabi.FA_MASK_WINDOW
         op.window_left = int(window_left)
     op.query_len = QL
+    if k_scales is not None or v_scales is not None:
+        if not fp8:
+            raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE, "k_scales / v_scales belong to FP8 caches")
+        _cabi.set_kv_scales(op, k_scales, v_scales, sh.num_kv_heads, sh.num_pool_blocks, query.device)
     # bytes are E5M2 as upstream fixes them (paged_attention_fp8_loop.cpp:43) unless the tensor says E4M3
     op.kv_fp8_format = _cabi.FA_FP8_E4M3 if key_cache.dtype == torch.float8_e4m3fn else _cabi.FA_FP8_E5M2
     op.stream = torch.cuda.current_stream(query.device).cuda_stream

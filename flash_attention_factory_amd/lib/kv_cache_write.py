@@ -8,12 +8,15 @@ call below produces the same bytes on the device: ``key``/``value`` are
 ``[blocks, block_size, kv_heads, head_size]`` views exactly as the ``paged_attention_*``
 modules take them, ``slot_mapping[n] = block * block_size + row`` (int64; a negative slot
 skips the token).  Returns the kernel time in microseconds as a one-element list, or
-``[]`` with ``timed=False`` (asynchronous on the current stream).
+``[]`` with ``timed=False`` (asynchronous on the current stream).  ``k_scales`` / ``v_scales``
+(fp32 device tensors ``[kv_heads]`` or ``[blocks, kv_heads]``) replace the scalar
+``fp8_scale``: a row is divided by the scale of its kv head, or of its destination block
+and kv head, before rounding.
 """
 from __future__ import annotations
 
 import ctypes
-from typing import List
+from typing import List, Optional
 
 import torch
 
@@ -21,7 +24,8 @@ from .. import _cabi
 
 
 def run(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
-        slot_mapping: torch.Tensor, fp8_scale: float = 1.0, *, timed: bool = True) -> List[float]:
+        slot_mapping: torch.Tensor, fp8_scale: float = 1.0, *, timed: bool = True,
+        k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None) -> List[float]:
     L = _cabi.load()
     if not key.is_cuda:
         raise RuntimeError("the KV-cache writer runs on the GPU only: `key` is not a device tensor")
@@ -55,6 +59,10 @@ def run(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_c
     elapsed = (ctypes.c_float * 2)(0.0, 0.0)
     op = _cabi.Options()
     op.fp8_scale = fp8_scale
+    if k_scales is not None or v_scales is not None:
+        if not fp8:
+            raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE, "k_scales / v_scales belong to FP8 pools")
+        _cabi.set_kv_scales(op, k_scales, v_scales, sh.num_kv_heads, sh.num_pool_blocks, key.device)
     op.stream = torch.cuda.current_stream(key.device).cuda_stream
     op.elapsed_us = ctypes.cast(elapsed, ctypes.POINTER(ctypes.c_float)) if timed else None
     with torch.cuda.device(key.device):

@@ -62,7 +62,9 @@ typedef struct fa_kv_cache_write_shape {
   int64_t num_pool_blocks;  /* blocks in each pool, > 0: slots outside the pool are skipped */
 } fa_kv_cache_write_shape;
 
-/* Of `options` this entry reads fp8_scale (E5M2 pools only; 0 means 1.0), stream,
+/* Of `options` this entry reads fp8_scale (FP8 pools only; 0 means 1.0), kv_scale_mode with
+ * k_scales / v_scales (FP8 pools only: the byte stored is the rounding of x * (1 / scale), the
+ * scale being that of the token's kv head or of its destination block and kv head), stream,
  * elapsed_us (1 float) and validate_only; the rest is ignored. */
 int32_t fa_kv_cache_write(const void *key, const void *value, void *key_cache, void *value_cache,
                           const int64_t *slot_mapping, const fa_kv_cache_write_shape *shape,

@@ -86,6 +86,15 @@ typedef enum fa_fp8_format { FA_FP8_E5M2 = 0, FA_FP8_E4M3 = 1 } fa_fp8_format;
  * query).  Opt-in: with mask_flags = 0 the entry points behave as upstream does. */
 typedef enum fa_mask { FA_MASK_ALIBI = 1, FA_MASK_SOFTCAP = 2, FA_MASK_WINDOW = 4 } fa_mask;
 
+/* Granularity of the dequantisation scales of an FP8 cache.  Upstream has one scalar for both
+ * caches (fp8_scale, paged_attention_kernel_fp8_loop.hpp:328-333,540-545): FA_KV_SCALE_TENSOR.
+ * The finer forms take separate K and V scales from device arrays:
+ *   FA_KV_SCALE_HEAD   k_scales, v_scales [num_kv_heads] fp32
+ *   FA_KV_SCALE_BLOCK  k_scales, v_scales [num_pool_blocks, num_kv_heads] fp32, one scale per
+ *                      physical block and kv head (num_pool_blocks must be given)
+ * K^ = dequant(K) * k_scale, V^ = dequant(V) * v_scale.  Scales must be finite and positive. */
+typedef enum fa_kv_scale { FA_KV_SCALE_TENSOR = 0, FA_KV_SCALE_HEAD = 1, FA_KV_SCALE_BLOCK = 2 } fa_kv_scale;
+
 /* Shapes and strides that upstream reads off the torch tensors
  * (paged_attention_loop.cpp:60-65) or fixes at compile time. */
 typedef struct fa_paged_attention_shape {
@@ -136,7 +145,11 @@ typedef struct fa_paged_attention_options {
                                  them) and token j sees the keys up to its own position -- upstream's
                                  causal rule, test_paged.py:79-80.  n * (num_heads / num_kv_heads)
                                  must not exceed 16 */
-  int32_t reserved;
+  int32_t kv_scale_mode;      /* FP8 entries and the KV-cache writer: fa_kv_scale.  0 = the scalar
+                                 fp8_scale as upstream; otherwise fp8_scale is ignored and the two
+                                 arrays below are read */
+  const float *k_scales;      /* device, fp32, shaped as kv_scale_mode says; NULL with mode 0 */
+  const float *v_scales;
 } fa_paged_attention_options;
 
 /* Single-pass kernel: one launch, no scratch. */

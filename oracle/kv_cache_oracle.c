@@ -16,9 +16,10 @@
  *                           every rounding boundary (tests/test_oracle_kv_cache.py).
  *   oracle_kv_cache_write   pinned against a torch index_put of cast tensors, both layouts,
  *                           skipped slots included.
- *   fp8_scale != 1          PARITY UNPINNED: upstream never quantises with a scale; the
- *                           reading implemented is byte = e5m2(fp32(x) * (1 / scale)),
- *                           rounded once.
+ *   fp8_scale != 1, scale   PARITY UNPINNED: upstream never quantises with a scale; the
+ *   arrays                  reading implemented is byte = fp8(fp32(x) * (1 / scale)),
+ *                           rounded once, the scale being the scalar, that of the kv head or
+ *                           that of the destination block and kv head.
  */
 #include <stdint.h>
 #include <string.h>
@@ -131,9 +132,13 @@ static void write_row(const uint16_t *src, void *cache, int64_t dst, const oracl
   }
 }
 
-ORACLE_API int oracle_kv_cache_write(const uint16_t *key, const uint16_t *value, void *key_cache,
-                                     void *value_cache, const int64_t *slot_mapping,
-                                     const oracle_kv_write *w) {
+/* k_scales / v_scales NULL: the scalar w->fp8_scale.  Otherwise the scale of a row is
+ * scales[b * scale_block_pitch + h]: per kv head with pitch 0, per destination block and kv
+ * head with pitch num_kv_heads.  The byte is the rounding of fp32(x) * (1.0f / scale). */
+ORACLE_API int oracle_kv_cache_write_scaled(const uint16_t *key, const uint16_t *value, void *key_cache,
+                                            void *value_cache, const int64_t *slot_mapping,
+                                            const float *k_scales, const float *v_scales,
+                                            int32_t scale_block_pitch, const oracle_kv_write *w) {
   const float inv = 1.0f / (w->fp8_scale != 0.f ? w->fp8_scale : 1.0f);
   const int64_t slots = w->num_pool_blocks * w->block_size;
   for (int64_t n = 0; n < w->num_tokens; ++n) {
@@ -143,9 +148,17 @@ ORACLE_API int oracle_kv_cache_write(const uint16_t *key, const uint16_t *value,
     for (int h = 0; h < w->num_kv_heads; ++h) {
       const int64_t src = n * w->src_token_stride + h * w->src_head_stride;
       const int64_t dst = b * w->kv_block_stride + t * w->kv_token_stride + h * w->kv_head_stride;
-      write_row(key + src, key_cache, dst, w, inv);
-      write_row(value + src, value_cache, dst, w, inv);
+      const float k_inv = k_scales ? 1.0f / k_scales[b * scale_block_pitch + h] : inv;
+      const float v_inv = v_scales ? 1.0f / v_scales[b * scale_block_pitch + h] : inv;
+      write_row(key + src, key_cache, dst, w, k_inv);
+      write_row(value + src, value_cache, dst, w, v_inv);
     }
   }
   return 0;
+}
+
+ORACLE_API int oracle_kv_cache_write(const uint16_t *key, const uint16_t *value, void *key_cache,
+                                     void *value_cache, const int64_t *slot_mapping,
+                                     const oracle_kv_write *w) {
+  return oracle_kv_cache_write_scaled(key, value, key_cache, value_cache, slot_mapping, NULL, NULL, 0, w);
 }

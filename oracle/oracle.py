@@ -79,6 +79,11 @@ def lib() -> ctypes.CDLL:
         L.oracle_attention_ref_masked.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32,
                                                   ctypes.c_int32, pp]
         L.oracle_attention_ref_masked.restype = ctypes.c_int
+        L.oracle_attention_ref_scaled.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32,
+                                                  ctypes.c_int32, P, P, ctypes.c_int32, pp]
+        L.oracle_attention_ref_scaled.restype = ctypes.c_int
+        L.oracle_kv_cache_write_scaled.argtypes = [P, P, P, P, P, P, P, ctypes.c_int32, P]
+        L.oracle_kv_cache_write_scaled.restype = ctypes.c_int
         L.oracle_kernel_loop.argtypes = [P, P, P, P, P, P, P, P, ctypes.c_int, pp]
         L.oracle_kernel_loop.restype = ctypes.c_int
         L.oracle_kernel_partition.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int, ctypes.c_int, pp]
@@ -148,12 +153,23 @@ def _bits_out(S, H, D, dtype):
     return torch.empty((S, H, D), dtype=dtype)
 
 
+def _scale_pitch(k_scales, v_scales, num_kv_heads, num_blocks) -> int:
+    """0 for per-head scales [Hk], Hk for per-block scales [NB, Hk]."""
+    for t in (k_scales, v_scales):
+        assert t is not None and t.dtype == torch.float32 and t.is_contiguous() and t.shape == k_scales.shape
+    if tuple(k_scales.shape) == (num_kv_heads,):
+        return 0
+    assert tuple(k_scales.shape) == (num_blocks, num_kv_heads), k_scales.shape
+    return num_kv_heads
+
+
 def attention_ref(query, key_cache, value_cache, block_tables, context_lens, *, scale, block_size,
                   kv_strides, num_kv_heads, sinks=None, fp8_scale=1.0, want_f32=False,
-                  alibi_slopes=None, softcap=0.0, window_left=-1):
+                  alibi_slopes=None, softcap=0.0, window_left=-1, k_scales=None, v_scales=None):
     """The upstream tests' PyTorch reference, restated (test_paged.py:40-168).  ``alibi_slopes``
     ([heads] fp32), ``softcap`` > 0 and ``window_left`` >= 0 switch on the score modifiers of
-    test_paged.py:92-110."""
+    test_paged.py:92-110.  ``k_scales`` / ``v_scales`` (fp32, ``[kv_heads]`` or
+    ``[blocks, kv_heads]``) replace ``fp8_scale`` for an FP8 cache."""
     query_len = 1
     q3 = query
     if query.dim() == 4:  # [S, query_len, H, D]: several query tokens per sequence, causal among themselves
@@ -165,7 +181,14 @@ def attention_ref(query, key_cache, value_cache, block_tables, context_lens, *, 
     S, H, D = q3.shape
     out = torch.zeros(query.shape, dtype=query.dtype)
     out32 = torch.zeros(query.shape, dtype=torch.float32)
-    if alibi_slopes is not None or softcap > 0 or window_left >= 0 or query_len > 1:
+    if k_scales is not None:
+        pitch = _scale_pitch(k_scales, v_scales, num_kv_heads, key_cache.shape[0])
+        rc = lib().oracle_attention_ref_scaled(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
+                                               _ptr(value_cache), _ptr(block_tables), _ptr(context_lens),
+                                               _ptr(sinks), _ptr(alibi_slopes), float(softcap), int(window_left),
+                                               int(query_len), _ptr(k_scales), _ptr(v_scales), pitch,
+                                               ctypes.byref(pr))
+    elif alibi_slopes is not None or softcap > 0 or window_left >= 0 or query_len > 1:
         if alibi_slopes is not None:
             assert alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and alibi_slopes.numel() == H
         rc = lib().oracle_attention_ref_masked(_ptr(out), _ptr(out32), _ptr(query), _ptr(key_cache),
@@ -253,7 +276,7 @@ def f32_to_e5m2(values: torch.Tensor) -> torch.Tensor:
 
 
 def kv_cache_write(key, value, key_cache, value_cache, slot_mapping, *, block_size, kv_strides,
-                   fp8_scale=1.0, e4m3=False):
+                   fp8_scale=1.0, e4m3=False, k_scales=None, v_scales=None):
     """Scatter the rows of `key`/`value` ([N, Hk, D], fp16/bf16) into the paged pools in place
     (the pool build of test_paged_fp8cache.py:171-203 as a per-token scatter)."""
     assert key.device.type == "cpu" and key.dim() == 3 and key.stride(2) == 1
@@ -273,6 +296,12 @@ def kv_cache_write(key, value, key_cache, value_cache, slot_mapping, *, block_si
     w.cache_dtype = (KV_E4M3 if (e4m3 or key_cache.dtype == torch.float8_e4m3fn) else KV_E5M2) if fp8 else KV_SAME_AS_Q
     w.num_pool_blocks = key_cache.shape[0]
     w.fp8_scale = fp8_scale
+    if k_scales is not None:
+        pitch = _scale_pitch(k_scales, v_scales, w.num_kv_heads, key_cache.shape[0])
+        lib().oracle_kv_cache_write_scaled(_ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache),
+                                           _ptr(slot_mapping), _ptr(k_scales), _ptr(v_scales), pitch,
+                                           ctypes.byref(w))
+        return
     lib().oracle_kv_cache_write(_ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache),
                                 _ptr(slot_mapping), ctypes.byref(w))
 

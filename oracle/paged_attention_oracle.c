@@ -179,20 +179,25 @@ typedef struct {
 /* Gather one (sequence, kv head)'s first n tokens of a cache into dense fp32
  * rows [n][D] (reference test_paged.py:184-193 does the same with fancy
  * indexing on the whole pool). */
-CLONES static void gather_rows(float *dst, const void *cache, const int32_t *table, int n,
-                               int kv_head, const oracle_problem *p) {
+/* `scales` NULL: every row is multiplied by p->fp8_scale.  Otherwise by
+ * scales[blk * scale_block_pitch + kv_head]: per-head scales with pitch 0, per physical
+ * block and kv head with pitch num_kv_heads (FP8 caches only). */
+CLONES static void gather_rows_scaled(float *dst, const void *cache, const int32_t *table, int n,
+                                      int kv_head, const oracle_problem *p, const float *scales,
+                                      int scale_block_pitch) {
   const int D = p->head_size, B = p->block_size;
   for (int t = 0; t < n; ++t) {
     int64_t blk = table[t / B];
+    const float mul = scales ? scales[blk * scale_block_pitch + kv_head] : p->fp8_scale;
     int64_t off = blk * p->kv_block_stride + (int64_t)(t % B) * p->kv_token_stride +
                   (int64_t)kv_head * p->kv_head_stride;
     float *row = dst + (size_t)t * D;
     if (p->kv_dtype == ORACLE_KV_E5M2) {
       const uint8_t *src = (const uint8_t *)cache + off;
-      for (int d = 0; d < D; ++d) row[d] = oracle_e5m2_to_f32(src[d]) * p->fp8_scale;
+      for (int d = 0; d < D; ++d) row[d] = oracle_e5m2_to_f32(src[d]) * mul;
     } else if (p->kv_dtype == ORACLE_KV_E4M3) {
       const uint8_t *src = (const uint8_t *)cache + off;
-      for (int d = 0; d < D; ++d) row[d] = oracle_e4m3_to_f32(src[d]) * p->fp8_scale;
+      for (int d = 0; d < D; ++d) row[d] = oracle_e4m3_to_f32(src[d]) * mul;
     } else {
       const uint16_t *src = (const uint16_t *)cache + off;
       if (p->q_dtype == ORACLE_Q_BF16)
@@ -201,6 +206,11 @@ CLONES static void gather_rows(float *dst, const void *cache, const int32_t *tab
         for (int d = 0; d < D; ++d) row[d] = oracle_f16_to_f32(src[d]);
     }
   }
+}
+
+static void gather_rows(float *dst, const void *cache, const int32_t *table, int n, int kv_head,
+                        const oracle_problem *p) {
+  gather_rows_scaled(dst, cache, table, n, kv_head, p, NULL, 0);
 }
 
 CLONES static float dot_f32(const float *a, const float *b, int n) {
@@ -249,6 +259,12 @@ typedef struct {
                         position -- upstream's causal rule, key j visible to query i iff
                         j <= i + seqlen_k - seqlen_q (test_paged.py:79-80 with the local mask
                         of :98-109).  1 = plain decode. */
+  /* Finer dequantisation scales of an FP8 cache (upstream has the one scalar fp8_scale):
+   * K^ = dequant(K) * k_scales[..], V^ = dequant(V) * v_scales[..], indexed
+   * [blk * scale_block_pitch + kv_head].  NULL = p->fp8_scale. */
+  const float *k_scales;
+  const float *v_scales;
+  int32_t scale_block_pitch;
 } oracle_masks;
 
 static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *query,
@@ -273,8 +289,10 @@ static int attention_ref_core(uint16_t *out, float *out_f32, const uint16_t *que
         failed = 1;
       } else {
         const int32_t *table = block_tables + (size_t)s * p->max_blocks_per_seq;
-        gather_rows(K, key_cache, table, n_all, kh, p);
-        gather_rows(V, value_cache, table, n_all, kh, p);
+        gather_rows_scaled(K, key_cache, table, n_all, kh, p, mk ? mk->k_scales : NULL,
+                           mk ? mk->scale_block_pitch : 0);
+        gather_rows_scaled(V, value_cache, table, n_all, kh, p, mk ? mk->v_scales : NULL,
+                           mk ? mk->scale_block_pitch : 0);
         for (int qg = 0; qg < QL * G; ++qg) {
           const int qt = qg / G, g = qg % G;
           const int n = n_all - QL + qt + 1; /* keys this query token sees */
@@ -332,7 +350,21 @@ ORACLE_API int oracle_attention_ref_masked(uint16_t *out, float *out_f32, const 
                                            const uint16_t *sinks, const float *alibi_slopes,
                                            float softcap, int32_t window_left, int32_t query_len,
                                            const oracle_problem *p) {
-  oracle_masks mk = {alibi_slopes, softcap, window_left, query_len};
+  oracle_masks mk = {alibi_slopes, softcap, window_left, query_len, NULL, NULL, 0};
+  return attention_ref_core(out, out_f32, query, key_cache, value_cache, block_tables, context_lens,
+                            sinks, p, &mk);
+}
+
+/* The same with per-head (scale_block_pitch 0) or per-block (scale_block_pitch num_kv_heads)
+ * K and V scales of an FP8 cache in place of p->fp8_scale. */
+ORACLE_API int oracle_attention_ref_scaled(uint16_t *out, float *out_f32, const uint16_t *query,
+                                           const void *key_cache, const void *value_cache,
+                                           const int32_t *block_tables, const int32_t *context_lens,
+                                           const uint16_t *sinks, const float *alibi_slopes,
+                                           float softcap, int32_t window_left, int32_t query_len,
+                                           const float *k_scales, const float *v_scales,
+                                           int32_t scale_block_pitch, const oracle_problem *p) {
+  oracle_masks mk = {alibi_slopes, softcap, window_left, query_len, k_scales, v_scales, scale_block_pitch};
   return attention_ref_core(out, out_f32, query, key_cache, value_cache, block_tables, context_lens,
                             sinks, p, &mk);
 }

@@ -29,14 +29,16 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 4
+    assert L.fa_paged_attention_abi_version() == 5
 
 
 def test_struct_layouts_match_header():
     # field order and sizes of the two structs as the header lays them out
     assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
     assert _cabi.Shape.kv_block_stride.offset == 32
-    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4
+    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4 + 8 + 8
+    assert _cabi.Options.kv_scale_mode.offset == 60
+    assert _cabi.Options.k_scales.offset == 64 and _cabi.Options.v_scales.offset == 72
     assert _cabi.Options.query_len.offset == 56
     assert _cabi.Options.mask_flags.offset == 48 and _cabi.Options.window_left.offset == 52
     assert _cabi.Options.elapsed_us.offset == 32
@@ -57,8 +59,10 @@ def _shape(**kw):
 
 
 def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0,
-          mask_flags=0, alibi=None, softcap=0.0, window_left=0, query_len=0):
+          mask_flags=0, alibi=None, softcap=0.0, window_left=0, query_len=0, scale_mode=0, k_scales=None,
+          v_scales=None):
     op = _cabi.Options()
+    op.kv_scale_mode, op.k_scales, op.v_scales = scale_mode, k_scales, v_scales
     op.query_len = query_len
     op.validate_only = 1
     op.kv_fp8_format = fp8_format
@@ -157,7 +161,7 @@ def test_workload_generators_are_deterministic():
     assert int(g.context_lens.min()) >= 319 and int(g.context_lens.max()) <= 339
 
 
-def _kv_write(L, ptr=0x1000, slots=0x1000, **kw):
+def _kv_write(L, ptr=0x1000, slots=0x1000, scale_mode=0, k_scales=None, v_scales=None, **kw):
     sh = _cabi.KvWriteShape()
     base = dict(num_tokens=4, num_kv_heads=2, head_size=128, block_size=16,
                 kv_block_stride=2 * 16 * 128, kv_token_stride=128, kv_head_stride=16 * 128,
@@ -168,6 +172,7 @@ def _kv_write(L, ptr=0x1000, slots=0x1000, **kw):
         setattr(sh, k, v)
     op = _cabi.Options()
     op.validate_only = 1
+    op.kv_scale_mode, op.k_scales, op.v_scales = scale_mode, k_scales, v_scales
     return L.fa_kv_cache_write(ptr, ptr, ptr, ptr, slots, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
 
 
@@ -186,3 +191,25 @@ def test_kv_cache_write_argument_checks(L):
     assert _kv_write(L, src_token_stride=100)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _kv_write(L, ptr=0x1008)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _kv_write(L, num_tokens=0)[0] == _cabi.FA_OK
+
+
+def test_kv_scale_argument_checks(L):
+    """Per-head / per-block scales: FP8 entries and the writer only, both arrays, a known pool size."""
+    HEAD, BLOCK = _cabi.FA_KV_SCALE_HEAD, _cabi.FA_KV_SCALE_BLOCK
+    for split in (False, True):
+        assert _call(L, split=split, fp8=True, scale_mode=HEAD, k_scales=0x1000, v_scales=0x2000)[0] == _cabi.FA_OK
+        assert _call(L, split=split, fp8=True, scale_mode=BLOCK, k_scales=0x1000, v_scales=0x2000)[0] == _cabi.FA_OK
+        rc, msg = _call(L, split=split, fp8=True, scale_mode=HEAD, k_scales=0x1000)
+        assert rc == _cabi.FA_ERR_NULL_POINTER and "v_scales" in msg
+        assert _call(L, split=split, fp8=True, scale_mode=3, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_ERR_BAD_SHAPE
+        assert _call(L, split=split, fp8=True, scale_mode=HEAD, k_scales=0x1002, v_scales=0x1000)[0] == _cabi.FA_ERR_BAD_SHAPE
+        rc, msg = _call(L, split=split, fp8=True, scale_mode=BLOCK, k_scales=0x1000, v_scales=0x1000,
+                        shape=_shape(num_pool_blocks=0))
+        assert rc == _cabi.FA_ERR_BAD_SHAPE and "num_pool_blocks" in msg
+        # a 16-bit cache has no scales: the fields are not read
+        assert _call(L, split=split, fp8=False, scale_mode=7)[0] == _cabi.FA_OK
+    assert _kv_write(L, scale_mode=HEAD, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_OK
+    assert _kv_write(L, scale_mode=BLOCK, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_OK
+    assert _kv_write(L, scale_mode=BLOCK, k_scales=0x1000)[0] == _cabi.FA_ERR_NULL_POINTER
+    assert _kv_write(L, scale_mode=9, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert _kv_write(L, scale_mode=9, cache_dtype=_cabi.FA_KV_CACHE_16BIT)[0] == _cabi.FA_OK
