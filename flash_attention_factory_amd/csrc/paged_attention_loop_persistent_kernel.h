@@ -236,6 +236,9 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     wa.reset(sink_raw);
     if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
     uint32_t next_sink = W::kNoSink;
+    if constexpr (EXT) {  // the sink goes with the item whether or not wavefront 0 has a chunk of it
+      if (has_next && !next_armed) next_sink = wa.load_sink(nxt.kvh, wave == 0);
+    }
     bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;

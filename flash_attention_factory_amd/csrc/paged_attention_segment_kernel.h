@@ -264,6 +264,10 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     wa.reset(sink_raw);
     if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
     uint32_t next_sink = W::kNoSink;
+    if constexpr (EXT) {
+      // a segment before the local window arms no wavefront, yet its partial carries the sink
+      if (has_next && !next_armed) next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+    }
     bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;

@@ -214,3 +214,27 @@ def test_write_then_attend_with_block_scales(oracle):
         _close(got, ref, kernel)
         err = (got.float().cpu() - exact).abs().max() / exact.abs().max()
         assert err < 0.1, (kernel, float(err))
+
+
+def test_block_scales_in_both_scheduling_forms(oracle):
+    """Per-block scales on a batch the persistent kernels take (100 sequences, several items per
+    work-group) and on one left to the grid form (300 sequences)."""
+    for S, seed in ((100, 71), (300, 72)):
+        gen = torch.Generator().manual_seed(seed)
+        lens = torch.randint(1, 1200, (S,), generator=gen)
+        lens[::11] = 0
+        w = W.make_test_shaped(batch_size=S, nheads=4, nheads_k=2, d=64, seqlen_k=1200, varlen=False, has_sinks=True,
+                               fp8=True, block_size=16, seed=seed, fp8_dtype=torch.float8_e4m3fn)
+        w.context_lens = lens.to(torch.int32)
+        w.partition_size = 256
+        NB = w.key_cache.shape[0]
+        ks, vs = _scales((NB, 2), seed, 0.2, 3.0), _scales((NB, 2), seed + 1, 0.01, 3.0)
+        ref = _ref(oracle, w, k_scales=ks, v_scales=vs)
+        wd = w.to(_dev())
+        live = lens > 0
+        for kernel in ("fp8_loop", "fp8_reduce"):
+            got = _call(wd, kernel, k_scales=ks.to(_dev()), v_scales=vs.to(_dev())).float().cpu()
+            assert (got[~live] == 0).all(), (S, kernel)
+            unit = ref[live].abs().max()
+            torch.testing.assert_close(got[live] / unit, ref[live] / unit, atol=ATOL, rtol=RTOL,
+                                       msg=lambda m: f"S={S} {kernel}: {m}")

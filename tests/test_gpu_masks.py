@@ -192,3 +192,32 @@ def test_query_tokens_head_major_e4m3(oracle):
     for kernel in ("fp8_loop", "fp8_reduce"):
         got = _call_multi(wd, query4.to(_dev()), kernel).float().cpu()
         torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel}: {m}")
+
+
+def test_extended_instances_in_both_scheduling_forms(oracle):
+    """Modifiers + two query tokens on a batch that the persistent kernels take (120 sequences,
+    several items per work-group, empty sequences in between) and on one they leave to the grid
+    form (300 sequences)."""
+    for S, seed in ((120, 31), (300, 32)):
+        gen = torch.Generator().manual_seed(seed)
+        lens = torch.randint(1, 1500, (S,), generator=gen)
+        lens[::9] = 0
+        lens[1] = 1                                    # shorter than the query block
+        w = W.make_config(0, num_seqs=S, pool_blocks=S * 94, lens=lens.tolist())     # D 64, G 1
+        w.partition_size = 256
+        w.sinks = torch.linspace(-2, 2, w.num_heads).to(w.query.dtype)
+        H = w.query.shape[1]
+        QL = 2
+        query4 = torch.randn(S, QL, H, 64, generator=gen).to(torch.float16)
+        alibi = torch.linspace(0.001, 0.03, H)
+        okw = dict(alibi_slopes=alibi, softcap=20.0, window_left=400)
+        ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                                   block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                                   sinks=w.sinks, want_f32=True, **okw)[1]
+        wd = w.to(_dev())
+        mods = dict(alibi_slopes=alibi.to(_dev()), softcap=20.0, apply_alibi=True, apply_softcap=True, window_left=400)
+        live = lens > 0
+        for kernel in ("loop", "reduce"):
+            got = _call_multi(wd, query4.to(_dev()), kernel, **dict(mods)).float().cpu()
+            assert (got[~live] == 0).all(), (S, kernel)          # empty sequences: rows untouched
+            torch.testing.assert_close(got[live], ref[live], atol=ATOL, rtol=RTOL, msg=lambda m: f"S={S} {kernel}: {m}")
