@@ -185,8 +185,8 @@ def _time_score_modifiers(built, steps, torch, W, runner, dev):
     visible = torch.clamp(w.context_lens, max=window_left + 1).sum().item()
     nbytes = visible * Hk * D * 2 * w.key_cache.element_size() + 2 * S * H * D * 2 + 4 * S + 4 * H \
         + sum(-(-min(int(c), window_left + 1) // B) for c in w.context_lens.tolist()) * 4
-    return dict(workload="config1 + soft-capping 30 + ALiBi + local window of 1024 keys (grid-form kernel)",
-                kernel="paged_attn_kernel<128, F16, kv16, loop, modifiers>", steps=steps, us_per_call=us,
+    return dict(workload="config1 + soft-capping 30 + ALiBi + local window of 1024 keys",
+                kernel="paged_attn_loop_persistent_kernel<128, F16, kv16, extended>", steps=steps, us_per_call=us,
                 algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
 
 
@@ -209,8 +209,8 @@ def _time_query_tokens(built, steps, torch, W, runner, dev, query_len=4):
             ts.append(t[0])
     us = float(torch.tensor(ts, dtype=torch.float64).mean())
     nbytes = w.algorithmic_bytes() + 2 * S * (query_len - 1) * H * D * 2
-    return dict(workload=f"config1 with {query_len} query tokens per sequence, causal (grid-form kernel)",
-                kernel="paged_attn_kernel<128, F16, kv16, loop, extended>", steps=steps, us_per_call=us,
+    return dict(workload=f"config1 with {query_len} query tokens per sequence, causal",
+                kernel="paged_attn_loop_persistent_kernel<128, F16, kv16, extended>", steps=steps, us_per_call=us,
                 algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
 
 
@@ -237,8 +237,8 @@ def _time_block_scales(built, steps, torch, W, runner, dev):
     us = float(torch.tensor(ts, dtype=torch.float64).mean())
     blocks = sum(-(-int(c) // B) for c in w.context_lens.tolist())
     nbytes = w.algorithmic_bytes() + blocks * Hk * 2 * 4
-    return dict(workload="config3 (E4M3 pools) with per-block K and V scales (grid-form kernel)",
-                kernel="paged_attn_kernel<128, F16, e4m3, loop, extended>", steps=steps, us_per_call=us,
+    return dict(workload="config3 (E4M3 pools) with per-block K and V scales",
+                kernel="paged_attn_loop_persistent_kernel<128, F16, e4m3, extended>", steps=steps, us_per_call=us,
                 algorithmic_bytes=nbytes, gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
 
 

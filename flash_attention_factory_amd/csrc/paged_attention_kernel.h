@@ -93,8 +93,9 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
 // MASKS: the extended instance.  It applies the score modifiers of p.mask_flags (soft-capping,
 // local window, ALiBi) and takes p.query_len query tokens per sequence, causal among
 // themselves (speculative decoding, chunked prefill): the MFMA columns are then (query token,
-// head) pairs.  Chunks that lie wholly before a sequence's window are skipped; a partition
-// of which a column sees nothing stores an empty partial for it (max -inf, sum 0, zeros).
+// head) pairs; an FP8 cache may bring per-head or per-block scales (p.kv_scale_mode).  Chunks
+// that lie wholly before a sequence's window are skipped; a partition of which a column sees
+// nothing stores an empty partial for it (max -inf, sum 0, zeros).
 template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC, bool MASKS = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {

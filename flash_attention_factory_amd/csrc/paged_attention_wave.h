@@ -68,9 +68,10 @@ constexpr int kScaleTensor = 0, kScaleHead = 1, kScaleBlock = 2;  // = fa_kv_sca
 // TPC: 16-token tiles per chunk (2 or 4).  One chunk is the unit of the software
 // pipeline; 4 tiles give an FP8 cache the same bytes in flight as 2 tiles of fp16.
 // KVF: cache format, kKv16 (elements of the query type), kKvE5M2 or kKvE4M3 (bytes).
-// EXT: the extended instance -- score modifiers and several query tokens per sequence
-// (p.mask_flags, p.query_len).  The MFMA columns then stand for (query token, head) pairs:
-// column i = query token i / G, head i % G of the kv head's group.
+// EXT: the extended instance -- score modifiers, several query tokens per sequence and
+// per-head or per-block scales of an FP8 cache (p.mask_flags, p.query_len, p.kv_scale_mode).
+// The MFMA columns then stand for (query token, head) pairs: column i = query token i / G,
+// head i % G of the kv head's group.
 template <int D, typename QT, int KVF, int TPC, bool STREAM, bool EXT = false>
 struct WaveAttn {
   static constexpr bool KV8 = KVF != kKv16;

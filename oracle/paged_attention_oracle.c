@@ -41,6 +41,11 @@
  *                            with an additive bias / mask and against plain torch ops for
  *                            the tanh cap (tests/test_oracle_masks.py).  Upstream's KERNELS
  *                            do not implement these (the code is commented out there).
+ *   oracle_attention_ref_scaled  per-head / per-block K and V scales of an FP8 cache:
+ *                            PARITY UNPINNED against upstream, which has nothing of the
+ *                            kind; the reading K^ = dequant(K)*k_scale, V^ = dequant(V)*v_scale
+ *                            is pinned against SDPA over tensors dequantised, scaled and
+ *                            gathered with torch indexing (tests/test_oracle_kv_scales.py).
  *   fp8_scale != 1           PARITY UNPINNED: the upstream tests only ever pass
  *                            1.0 (test_paged_fp8cache.py:489,510); the reading
  *                            implemented is K^ = dequant(K)*s, V^ = dequant(V)*s.
