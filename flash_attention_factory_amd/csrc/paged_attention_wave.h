@@ -336,7 +336,14 @@ struct WaveAttn {
                                         const TileScales *ts = nullptr) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
     float t[NT];
-    if constexpr (MASKS) {
+    if (MASKS && p.mask_flags == 0 && p.query_len <= 1) {
+      // only scales asked for the extended instance: plain scores with the tiles' own scale
+      float k2[TPC];
+#pragma unroll
+      for (int tl = 0; tl < TPC; ++tl) k2[tl] = ts->k[tl] * kLog2e;
+#pragma unroll
+      for (int e = 0; e < NT; ++e) t[e] = s.v[e >> 2][e & 3] * k2[e >> 2];
+    } else if constexpr (MASKS) {
       const bool cap = p.mask_flags & kMaskSoftcap;
       const float inv_cap2 = 2.0f * kLog2e / p.softcap;  // exp(2x/cap) = exp2(x * inv_cap2)
       const int first_visible = (p.mask_flags & kMaskWindow) ? col_last - p.window_left : 0;
