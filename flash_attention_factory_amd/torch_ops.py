@@ -18,6 +18,13 @@ recorded into a HIP graph (``torch.cuda.graph``) and replayed.
     torch.ops.fa_amd.paged_attention_fp8_reduce(..., scale, fp8_scale, partition_size, sinks)
     torch.ops.fa_amd.kv_cache_write(key, value, key_cache, value_cache, slot_mapping, fp8_scale)
 
+Further optional arguments, all off by default: ``alibi_slopes`` (fp32 ``[heads]``), ``softcap``
+(> 0) and ``window_left`` (>= 0) apply the score modifiers -- here a modifier that is passed is
+applied, unlike ``lib.*.run``, which mirrors upstream in taking and ignoring slopes and cap; the
+FP8 operators and ``kv_cache_write`` take ``k_scales`` / ``v_scales`` (fp32 ``[kv_heads]`` or
+``[blocks, kv_heads]``) in place of the scalar ``fp8_scale``.  ``query`` / ``out`` may be
+``[seqs, query_len, heads, head_size]``: several causal query tokens per sequence.
+
 Caches are ``[blocks, block_size, kv_heads, head_size]`` views as in ``lib.*.run``; every
 output is an argument the operator mutates, nothing is allocated.  Importing this module
 registers the operators; there is no CPU implementation.
@@ -37,36 +44,47 @@ _NS = "fa_amd"
 
 
 def _group(query: Tensor, key_cache: Tensor) -> int:
-    return query.size(1) // key_cache.size(2)
+    return query.size(-2) // key_cache.size(2)
+
+
+def _modifiers(alibi_slopes: Optional[Tensor], softcap: float, window_left: int) -> dict:
+    return dict(apply_alibi=alibi_slopes is not None, apply_softcap=softcap > 0.0,
+                window_left=window_left if window_left >= 0 else None)
 
 
 @torch.library.custom_op(f"{_NS}::paged_attention_loop", mutates_args=("out",), device_types="cuda")
 def paged_attention_loop(out: Tensor, query: Tensor, key_cache: Tensor, value_cache: Tensor,
                          block_tables: Tensor, context_lens: Tensor, scale: float,
-                         sinks: Optional[Tensor] = None) -> None:
+                         sinks: Optional[Tensor] = None, alibi_slopes: Optional[Tensor] = None,
+                         softcap: float = 0.0, window_left: int = -1) -> None:
     _loop.run(None, None, None, out, None, query, key_cache, value_cache, block_tables, context_lens,
-              _group(query, key_cache), scale, key_cache.size(1), 0, None, sinks, 0.0, timed=False)
+              _group(query, key_cache), scale, key_cache.size(1), 0, alibi_slopes, sinks, softcap, timed=False,
+              **_modifiers(alibi_slopes, softcap, window_left))
 
 
 @torch.library.custom_op(f"{_NS}::paged_attention_fp8_loop", mutates_args=("out",), device_types="cuda")
 def paged_attention_fp8_loop(out: Tensor, query: Tensor, key_cache: Tensor, value_cache: Tensor,
                              block_tables: Tensor, context_lens: Tensor, scale: float, fp8_scale: float,
-                             sinks: Optional[Tensor] = None) -> None:
+                             sinks: Optional[Tensor] = None, alibi_slopes: Optional[Tensor] = None,
+                             softcap: float = 0.0, window_left: int = -1, k_scales: Optional[Tensor] = None,
+                             v_scales: Optional[Tensor] = None) -> None:
     _fp8_loop.run(None, None, None, out, None, query, key_cache, value_cache, block_tables, context_lens,
-                  _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, None, sinks, 0.0,
-                  timed=False)
+                  _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, alibi_slopes, sinks, softcap,
+                  timed=False, k_scales=k_scales, v_scales=v_scales, **_modifiers(alibi_slopes, softcap, window_left))
 
 
 @torch.library.custom_op(f"{_NS}::paged_attention_reduce",
                          mutates_args=("out", "exp_sums", "max_logits", "tmp_out"), device_types="cuda")
 def paged_attention_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tmp_out: Tensor, query: Tensor,
                            key_cache: Tensor, value_cache: Tensor, block_tables: Tensor, context_lens: Tensor,
-                           scale: float, partition_size: int = 0, sinks: Optional[Tensor] = None) -> None:
+                           scale: float, partition_size: int = 0, sinks: Optional[Tensor] = None,
+                           alibi_slopes: Optional[Tensor] = None, softcap: float = 0.0,
+                           window_left: int = -1) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
     _reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
-                context_lens, _group(query, key_cache), scale, key_cache.size(1), 0, None, sinks, 0.0,
-                partition_size=partition_size, timed=False)
+                context_lens, _group(query, key_cache), scale, key_cache.size(1), 0, alibi_slopes, sinks, softcap,
+                partition_size=partition_size, timed=False, **_modifiers(alibi_slopes, softcap, window_left))
 
 
 @torch.library.custom_op(f"{_NS}::paged_attention_fp8_reduce",
@@ -74,18 +92,23 @@ def paged_attention_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tm
 def paged_attention_fp8_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tmp_out: Tensor, query: Tensor,
                                key_cache: Tensor, value_cache: Tensor, block_tables: Tensor,
                                context_lens: Tensor, scale: float, fp8_scale: float, partition_size: int = 0,
-                               sinks: Optional[Tensor] = None) -> None:
+                               sinks: Optional[Tensor] = None, alibi_slopes: Optional[Tensor] = None,
+                               softcap: float = 0.0, window_left: int = -1, k_scales: Optional[Tensor] = None,
+                               v_scales: Optional[Tensor] = None) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
     _fp8_reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
-                    context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, None, sinks,
-                    0.0, partition_size=partition_size, timed=False)
+                    context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, alibi_slopes,
+                    sinks, softcap, partition_size=partition_size, timed=False, k_scales=k_scales,
+                    v_scales=v_scales, **_modifiers(alibi_slopes, softcap, window_left))
 
 
 @torch.library.custom_op(f"{_NS}::kv_cache_write", mutates_args=("key_cache", "value_cache"), device_types="cuda")
 def kv_cache_write(key: Tensor, value: Tensor, key_cache: Tensor, value_cache: Tensor, slot_mapping: Tensor,
-                   fp8_scale: float = 1.0) -> None:
-    _kv_cache_write.run(key, value, key_cache, value_cache, slot_mapping, fp8_scale, timed=False)
+                   fp8_scale: float = 1.0, k_scales: Optional[Tensor] = None,
+                   v_scales: Optional[Tensor] = None) -> None:
+    _kv_cache_write.run(key, value, key_cache, value_cache, slot_mapping, fp8_scale, timed=False,
+                        k_scales=k_scales, v_scales=v_scales)
 
 
 # Shape propagation for tracing: every operator only writes into its arguments.

@@ -113,3 +113,60 @@ def test_decode_step_in_a_hip_graph():
         assert torch.equal(graphed["kc"].view(torch.uint8), eager["kc"].view(torch.uint8)), f"key pool, replay {replay}"
         a, b = eager["loop"].out.float(), eager["split"].out.float()
         assert (a - b).abs().max().item() <= 2.0 ** -9 * a.abs().max().item() + 1e-5
+
+
+def test_operators_with_modifiers_query_tokens_and_block_scales(oracle):
+    """The optional arguments of the operators against the oracle, eagerly and as a HIP graph
+    replayed with fresh inputs: window + ALiBi + soft-capping, three query tokens per sequence,
+    E4M3 pools with per-block scales."""
+    from flash_attention_factory_amd import torch_ops  # noqa: F401
+    dev = _dev()
+    ops = torch.ops.fa_amd
+    w = W.make_test_shaped(batch_size=3, nheads=8, nheads_k=2, d=128, seqlen_k=900, varlen=True, has_sinks=True,
+                           fp8=True, block_size=16, seed=81, fp8_dtype=torch.float8_e4m3fn)
+    S, H, D, QL = 3, 8, 128, 3
+    NB = w.key_cache.shape[0]
+    g = torch.Generator().manual_seed(2)
+    ks = torch.rand((NB, 2), generator=g) * 2 + 0.2
+    vs = torch.rand((NB, 2), generator=g) * 2 + 0.2
+    alibi = torch.linspace(0.002, 0.02, H)
+    NP = -(-int(w.context_lens.max()) // 512)
+    wd = w.to(dev)
+    query = torch.zeros((S, QL, H, D), dtype=torch.float16, device=dev)
+    out_a, out_b = torch.zeros_like(query), torch.zeros_like(query)
+    es = torch.zeros((S * QL, H, NP), dtype=torch.float32, device=dev)
+    ml, tmp = torch.zeros_like(es), torch.zeros((S * QL, H, NP, D), dtype=torch.float32, device=dev)
+    ks_d, vs_d, alibi_d = ks.to(dev), vs.to(dev), alibi.to(dev)
+
+    def step():
+        ops.paged_attention_fp8_loop(out_a, query, wd.key_cache, wd.value_cache, wd.block_tables, wd.context_lens,
+                                     w.scale, 1.0, wd.sinks, alibi_d, 15.0, 500, ks_d, vs_d)
+        ops.paged_attention_fp8_reduce(out_b, es, ml, tmp, query, wd.key_cache, wd.value_cache, wd.block_tables,
+                                       wd.context_lens, w.scale, 1.0, 512, wd.sinks, alibi_d, 15.0, 500, ks_d, vs_d)
+
+    def check(q_cpu, what):
+        ref = oracle.attention_ref(q_cpu, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                                   block_size=16, kv_strides=w.kv_strides(), num_kv_heads=2, sinks=w.sinks,
+                                   want_f32=True, alibi_slopes=alibi, softcap=15.0, window_left=500,
+                                   k_scales=ks, v_scales=vs)[1]
+        unit = ref.abs().max()
+        for name, out in (("loop", out_a), ("split", out_b)):
+            torch.testing.assert_close(out.float().cpu() / unit, ref / unit, atol=1e-2, rtol=1e-2,
+                                       msg=lambda m: f"{what} {name}: {m}")
+
+    q0 = torch.randn((S, QL, H, D), generator=g).to(torch.float16)
+    query.copy_(q0)
+    step()                      # eager (and warm-up for the capture)
+    torch.cuda.synchronize()
+    check(q0, "eager")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for it in range(3):
+        qn = torch.randn((S, QL, H, D), generator=g).to(torch.float16)
+        query.copy_(qn)
+        out_a.zero_(); out_b.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check(qn, f"replay {it}")
