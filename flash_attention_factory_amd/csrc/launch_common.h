@@ -13,6 +13,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <algorithm>
+
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
 #include "paged_attention_loop_persistent_kernel.h"
@@ -48,6 +50,11 @@ inline int ilog2(int32_t v) {
   while ((1 << s) < v) ++s;
   return s;
 }
+
+// Query tokens per sequence an extended call may bring.  The 16 MFMA columns hold
+// 16 / (heads per kv head) of them at a time; a call with more runs as several launches, each
+// reading K and V once.
+constexpr int kMaxQueryLen = 64;
 
 struct Resolved {
   int32_t group;
@@ -144,9 +151,8 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
     return fail(FA_ERR_BAD_SHAPE, "FA_MASK_WINDOW needs window_left >= 0");
   r->query_len = (o && o->query_len > 1) ? o->query_len : 1;
   if (o && o->query_len < 0) return fail(FA_ERR_BAD_SHAPE, "query_len must be >= 0");
-  if ((int64_t)r->query_len * r->group > kMaxGroup)
-    return fail(FA_ERR_UNSUPPORTED_GROUP, "query_len %d x %d queries per kv head exceeds %d", r->query_len,
-                r->group, kMaxGroup);
+  if (r->query_len > kMaxQueryLen)
+    return fail(FA_ERR_BAD_SHAPE, "query_len %d exceeds %d", r->query_len, kMaxQueryLen);
   if ((int64_t)s->num_seqs * r->query_len > 65535)
     return fail(FA_ERR_BAD_SHAPE, "num_seqs x query_len %lld exceeds the grid limit 65535",
                 (long long)s->num_seqs * r->query_len);
@@ -197,6 +203,8 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.softcap = r.softcap;
   p.window_left = r.window_left;
   p.query_len = r.query_len;
+  p.query_first = 0;
+  p.query_count = std::min(r.query_len, kMaxGroup / r.group);
   p.out_scale = r.fp8_scale;
   p.kv_scale_mode = r.kv_scale_mode;
   p.k_scales = r.k_scales;
@@ -266,6 +274,15 @@ class KernelTimer {
     if (e != hipSuccess) return e;
     hipExtLaunchKernelGGL(kernel, grid, block, 0, stream_, events()[2 * slot], events()[2 * slot + 1], 0, prm);
     return hipGetLastError();
+  }
+
+  // Time of the launch last made in `slot`, ADDED to *us: a call that makes several launches
+  // in a slot reads after each of them.
+  hipError_t accumulate(int slot, float *us) {
+    float one = 0.f;
+    const hipError_t e = read(slot, &one);
+    *us += one;
+    return e;
   }
 
   hipError_t read(int slot, float *us) {

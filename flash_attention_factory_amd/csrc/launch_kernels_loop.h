@@ -23,41 +23,48 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
                                         const fa_paged_attention_shape &shape, const Resolved &r) {
   constexpr bool KV8 = KVF != kKv16;
   constexpr int NW = WavesPerGroup<false>::value;
-  const PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
-                                        block_tables, context_lens, scale, shape, r);
+  PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
+                                  block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
   const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
-  if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
-      max_ctx < kLoopPersistentMaxContext) {
-    // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
-    // sequences first, with the next item's first loads issued before each merge.
-    constexpr int PW = PersistentLoop<KV8>::waves;
-    auto plain = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                   Pipeline<KV8>::tiles_per_chunk, false>;
-    auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                      Pipeline<KV8>::tiles_per_chunk, true>;
-    auto kernel = ext ? extended : plain;
-    int resident = 0;
-    FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
-    const dim3 grid((unsigned)std::min<int64_t>(resident, items));
-    FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
-  } else if (ext) {
-    const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
-    FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
-                          Pipeline<KV8>::tiles_per_chunk, true>,
-        grid, dim3(NW * 64), 0, p));
-  } else {
-    const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
-    FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
-                          Pipeline<KV8>::tiles_per_chunk>,
-        grid, dim3(NW * 64), 0, p));
+  float total_us = 0.f;
+  // One launch per group of query tokens that fit the 16 MFMA columns (one launch for decode).
+  for (int q0 = 0; q0 < r.query_len; q0 += p.query_count) {
+    p.query_first = q0;
+    p.query_count = std::min(p.query_count, r.query_len - q0);
+    if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
+        max_ctx < kLoopPersistentMaxContext) {
+      // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
+      // sequences first, with the next item's first loads issued before each merge.
+      constexpr int PW = PersistentLoop<KV8>::waves;
+      auto plain = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk, false>;
+      auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                        Pipeline<KV8>::tiles_per_chunk, true>;
+      auto kernel = ext ? extended : plain;
+      int resident = 0;
+      FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
+      const dim3 grid((unsigned)std::min<int64_t>(resident, items));
+      FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
+    } else if (ext) {
+      const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+      FA_HIP_CHECK(timer.launch(
+          paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
+                            Pipeline<KV8>::tiles_per_chunk, true>,
+          grid, dim3(NW * 64), 0, p));
+    } else {
+      const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+      FA_HIP_CHECK(timer.launch(
+          paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
+                            Pipeline<KV8>::tiles_per_chunk>,
+          grid, dim3(NW * 64), 0, p));
+    }
+    if (r.elapsed_us) FA_HIP_CHECK(timer.accumulate(0, &total_us));
   }
-  if (r.elapsed_us) FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
+  if (r.elapsed_us) r.elapsed_us[0] = total_us;
   return FA_OK;
 }
 

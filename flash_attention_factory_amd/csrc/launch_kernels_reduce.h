@@ -24,8 +24,8 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
                                       const fa_paged_attention_shape &shape, const Resolved &r) {
   constexpr bool KV8 = KVF != kKv16;
   constexpr int NW = WavesPerGroup<true>::value;
-  const PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache,
-                                        value_cache, block_tables, context_lens, scale, shape, r);
+  PagedAttnParams p = make_params(tmp_out, exp_sums, max_logits, query, key_cache, value_cache,
+                                  block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
   // kernel 1.  Segment form when the batch fits it: as many multi-wavefront work-groups as
   // the GPU keeps resident share out segments of several partitions.  Otherwise one
@@ -34,33 +34,41 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   int segment_groups = 0;  // > 0: the segment kernel ran with that many work-groups
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
-  if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
-      (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
-    // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
-    constexpr int SW = SegmentSplit<KV8>::waves;
-    auto plain = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                           Pipeline<KV8>::tiles_per_chunk, false>;
-    auto extended = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                              Pipeline<KV8>::tiles_per_chunk, true>;
-    auto kernel = ext ? extended : plain;
-    int resident = 0;
-    FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
-    const int64_t max_items =
-        (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
-    segment_groups = (int)std::min<int64_t>(resident, max_items);
-    FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
-  } else if (ext) {
-    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
-    FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
-                          Pipeline<KV8>::tiles_per_chunk, true>,
-        grid, dim3(NW * 64), 0, p));
-  } else {
-    const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
-    FA_HIP_CHECK(timer.launch(
-        paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
-                          Pipeline<KV8>::tiles_per_chunk>,
-        grid, dim3(NW * 64), 0, p));
+  float attention_us = 0.f;
+  // One launch per group of query tokens that fit the 16 MFMA columns (one launch for decode);
+  // every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
+  for (int q0 = 0; q0 < r.query_len; q0 += p.query_count) {
+    p.query_first = q0;
+    p.query_count = std::min(p.query_count, r.query_len - q0);
+    if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
+        (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
+      // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
+      constexpr int SW = SegmentSplit<KV8>::waves;
+      auto plain = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                             Pipeline<KV8>::tiles_per_chunk, false>;
+      auto extended = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                                Pipeline<KV8>::tiles_per_chunk, true>;
+      auto kernel = ext ? extended : plain;
+      int resident = 0;
+      FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
+      const int64_t max_items =
+          (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
+      segment_groups = (int)std::min<int64_t>(resident, max_items);
+      FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
+    } else if (ext) {
+      const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+      FA_HIP_CHECK(timer.launch(
+          paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
+                            Pipeline<KV8>::tiles_per_chunk, true>,
+          grid, dim3(NW * 64), 0, p));
+    } else {
+      const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+      FA_HIP_CHECK(timer.launch(
+          paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
+                            Pipeline<KV8>::tiles_per_chunk>,
+          grid, dim3(NW * 64), 0, p));
+    }
+    if (r.elapsed_us) FA_HIP_CHECK(timer.accumulate(0, &attention_us));
   }
 
   // kernel 2: one wavefront per (head, sequence)
@@ -88,7 +96,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
     else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, false>, rgrid, dim3(256), 1, rp));
   }
   if (r.elapsed_us) {
-    FA_HIP_CHECK(timer.read(0, &r.elapsed_us[0]));
+    r.elapsed_us[0] = attention_us;
     FA_HIP_CHECK(timer.read(1, &r.elapsed_us[1]));
   }
   return FA_OK;

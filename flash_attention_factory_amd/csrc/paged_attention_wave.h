@@ -55,6 +55,8 @@ struct PagedAttnParams {
   int32_t window_left;
   int32_t mask_flags;           // kMaskAlibi | kMaskSoftcap | kMaskWindow
   int32_t query_len;            // query tokens per sequence (1 = plain decode)
+  int32_t query_first;          // of those, the launch at hand covers tokens query_first ..
+  int32_t query_count;          // query_first + query_count - 1 (query_count * group <= 16)
   // finer dequantisation scales of an FP8 cache, read only by the extended instances.  With a
   // mode other than kScaleTensor score_scale is the bare softmax scale and out_scale is 1.
   int32_t kv_scale_mode;        // kScaleTensor / kScaleHead / kScaleBlock
@@ -70,8 +72,9 @@ constexpr int kScaleTensor = 0, kScaleHead = 1, kScaleBlock = 2;  // = fa_kv_sca
 // KVF: cache format, kKv16 (elements of the query type), kKvE5M2 or kKvE4M3 (bytes).
 // EXT: the extended instance -- score modifiers, several query tokens per sequence and
 // per-head or per-block scales of an FP8 cache (p.mask_flags, p.query_len, p.kv_scale_mode).
-// The MFMA columns then stand for (query token, head) pairs: column i = query token i / G,
-// head i % G of the kv head's group.
+// The MFMA columns then stand for (query token, head) pairs: column i = query token
+// p.query_first + i / G, head i % G of the kv head's group; a launch covers the p.query_count
+// tokens that fit the 16 columns, the host launches once per such group of tokens.
 template <int D, typename QT, int KVF, int TPC, bool STREAM, bool EXT = false>
 struct WaveAttn {
   static constexpr bool KV8 = KVF != kKv16;
@@ -124,9 +127,10 @@ struct WaveAttn {
   __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
       : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {
     if constexpr (EXT) {
-      col_q = i / prm.group;
-      col_g = i - col_q * prm.group;
-      col_valid = i < prm.group * prm.query_len;
+      const int q = i / prm.group;
+      col_g = i - q * prm.group;
+      col_q = prm.query_first + q;
+      col_valid = q < prm.query_count;
     } else {
       col_g = i;
       col_valid = i < prm.group;
@@ -176,7 +180,7 @@ struct WaveAttn {
   // First chunk that holds a key some query token of the item sees (local window), at least c_begin.
   __device__ __forceinline__ int first_visible_chunk(int ctx, int c_begin) const {
     if (!(p.mask_flags & kMaskWindow)) return c_begin;
-    return max(c_begin, max(0, ctx - p.query_len - p.window_left) / CT);
+    return max(c_begin, max(0, ctx - p.query_len + p.query_first - p.window_left) / CT);
   }
 
   // EXT: multipliers of a chunk's tiles (uniform over the item unless the scales are per block).

@@ -102,7 +102,10 @@ def test_score_modifier_arguments(L):
 
 def test_query_len_limits(L):
     assert _call(L, query_len=4)[0] == _cabi.FA_OK                      # group 4 x 4 tokens = 16 columns
-    assert _call(L, query_len=5)[0] == _cabi.FA_ERR_UNSUPPORTED_GROUP
+    assert _call(L, query_len=5)[0] == _cabi.FA_OK                      # two launches: 4 tokens, then 1
+    assert _call(L, query_len=64)[0] == _cabi.FA_OK
+    rc, msg = _call(L, query_len=65)
+    assert rc == _cabi.FA_ERR_BAD_SHAPE and "query_len" in msg
     assert _call(L, split=True, query_len=2)[0] == _cabi.FA_OK
     assert _call(L, query_len=-1)[0] == _cabi.FA_ERR_BAD_SHAPE
 

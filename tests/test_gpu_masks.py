@@ -221,3 +221,28 @@ def test_extended_instances_in_both_scheduling_forms(oracle):
             got = _call_multi(wd, query4.to(_dev()), kernel, **dict(mods)).float().cpu()
             assert (got[~live] == 0).all(), (S, kernel)          # empty sequences: rows untouched
             torch.testing.assert_close(got[live], ref[live], atol=ATOL, rtol=RTOL, msg=lambda m: f"S={S} {kernel}: {m}")
+
+
+@pytest.mark.parametrize("QL,nheads,nheads_k", [(4, 16, 2), (7, 8, 2), (33, 2, 2), (3, 16, 1)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_more_query_tokens_than_the_mfma_columns_hold(oracle, QL, nheads, nheads_k, fp8):
+    """QL x (heads per kv head) beyond 16: the call runs as several launches, each covering the
+    query tokens that fit the 16 columns (8+8 heads x 2+2 tokens; 4 heads x 4+3 tokens; 16 + 16 + 1
+    tokens of one head; 16 heads x 1+1+1 tokens), with a window and ALiBi placed per token."""
+    w = W.make_test_shaped(batch_size=3, nheads=nheads, nheads_k=nheads_k, d=128, seqlen_k=1100, varlen=True,
+                           has_sinks=True, fp8=fp8, seed=19)
+    w.context_lens[0] = QL - 1             # the first query token lies before key 0
+    w.context_lens[1] = 512 + 2
+    g = torch.Generator().manual_seed(5)
+    query4 = torch.randn(3, QL, nheads, 128, generator=g).to(torch.float16)
+    alibi = torch.linspace(0.002, 0.02, nheads)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, fp8_scale=w.fp8_scale, want_f32=True, alibi_slopes=alibi,
+                               window_left=300)[1]
+    wd = w.to(_dev())
+    for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+        got = _call_multi(wd, query4.to(_dev()), kernel, alibi_slopes=alibi.to(_dev()), apply_alibi=True,
+                          window_left=300).float().cpu()
+        assert torch.isfinite(got).all(), kernel
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel} QL={QL}: {m}")
