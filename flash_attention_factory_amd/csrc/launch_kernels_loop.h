@@ -13,14 +13,16 @@
 
 namespace fa {
 
-// One launch, grid (kv heads, 1, sequences), NW wavefronts per work-group.
+// The launches of one batch that a single kernel launch can take: persistent form for up to
+// kLoopPersistentMaxSeqs sequences, else grid (kv heads, 1, sequences) with NW wavefronts per
+// work-group.  Kernel time is ADDED to *total_us when the call is timed.
 // KVF selects the cache format: 16-bit, or E5M2 / E4M3 bytes (launch_kernels_fp8_loop.h).
 template <int HEAD_SIZE, typename QT, int KVF>
-inline fa_status launch_paged_attn_loop(void *out, const void *query, const void *key_cache,
-                                        const void *value_cache, const int32_t *block_tables,
-                                        const int32_t *context_lens, float scale,
-                                        int32_t /*max_context_len: validation only*/,
-                                        const fa_paged_attention_shape &shape, const Resolved &r) {
+inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, const void *key_cache,
+                                              const void *value_cache, const int32_t *block_tables,
+                                              const int32_t *context_lens, float scale,
+                                              const fa_paged_attention_shape &shape, const Resolved &r,
+                                              float *total_us_out) {
   constexpr bool KV8 = KVF != kKv16;
   constexpr int NW = WavesPerGroup<false>::value;
   PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
@@ -63,6 +65,44 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
           grid, dim3(NW * 64), 0, p));
     }
     if (r.elapsed_us) FA_HIP_CHECK(timer.accumulate(0, &total_us));
+  }
+  *total_us_out += total_us;
+  return FA_OK;
+}
+
+// Whether the persistent kernel takes batches of this shape at all (given few enough sequences).
+inline bool loop_persistent_fits(const fa_paged_attention_shape &shape) {
+  return kUsePersistentLoop && shape.num_pool_blocks > 0 &&
+         (int64_t)shape.max_blocks_per_seq * shape.block_size < kLoopPersistentMaxContext;
+}
+
+// A batch of more sequences than the persistent kernel ranks is cut into equal sub-batches,
+// one persistent launch each, where that beats the grid form (PersistentLoop::sub_batches).
+template <int HEAD_SIZE, typename QT, int KVF>
+inline fa_status launch_paged_attn_loop(void *out, const void *query, const void *key_cache,
+                                        const void *value_cache, const int32_t *block_tables,
+                                        const int32_t *context_lens, float scale,
+                                        int32_t /*max_context_len: validation only*/,
+                                        const fa_paged_attention_shape &shape, const Resolved &r) {
+  float total_us = 0.f;
+  if (PersistentLoop<(KVF != kKv16)>::sub_batches && loop_persistent_fits(shape) &&
+      shape.num_seqs > kLoopPersistentMaxSeqs) {
+    const int pieces = (shape.num_seqs + kLoopPersistentMaxSeqs - 1) / kLoopPersistentMaxSeqs;
+    const int per = (shape.num_seqs + pieces - 1) / pieces;
+    const int64_t row_bytes = (int64_t)r.query_len * shape.num_heads * shape.head_size * 2;  // of query and out
+    for (int s0 = 0; s0 < shape.num_seqs; s0 += per) {
+      fa_paged_attention_shape sub = shape;
+      sub.num_seqs = std::min(per, shape.num_seqs - s0);
+      const fa_status st = launch_paged_attn_loop_batch<HEAD_SIZE, QT, KVF>(
+          reinterpret_cast<char *>(out) + s0 * row_bytes, reinterpret_cast<const char *>(query) + s0 * row_bytes,
+          key_cache, value_cache, block_tables + (int64_t)s0 * shape.max_blocks_per_seq, context_lens + s0, scale,
+          sub, r, &total_us);
+      if (st != FA_OK) return st;
+    }
+  } else {
+    const fa_status st = launch_paged_attn_loop_batch<HEAD_SIZE, QT, KVF>(
+        out, query, key_cache, value_cache, block_tables, context_lens, scale, shape, r, &total_us);
+    if (st != FA_OK) return st;
   }
   if (r.elapsed_us) r.elapsed_us[0] = total_us;
   return FA_OK;

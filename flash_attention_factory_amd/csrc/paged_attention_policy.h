@@ -120,6 +120,11 @@ template <bool kKV8>
 struct PersistentLoop {
   static constexpr int waves = kKV8 ? FA_PLOOP_WAVES_FP8 : FA_PLOOP_WAVES;
   static constexpr int occ = kKV8 ? FA_PLOOP_OCC_FP8 : FA_PLOOP_OCC;
+  // Batches beyond what the kernel ranks in one launch: cut into sub-batches (one persistent
+  // launch each), or left to the grid form?  Measured with 512 sequences of 512-2048 tokens:
+  // 16-bit caches 82.4 % of peak in sub-batches against 80.2 % in the grid form; FP8 caches,
+  // whose launches are half as long and so pay the fixed costs twice, 77.8 % against 79.6 %.
+  static constexpr bool sub_batches = !kKV8;
 };
 
 // ---- reduce kernel ---------------------------------------------------------------------

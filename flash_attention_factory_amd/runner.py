@@ -50,9 +50,11 @@ def alloc_buffers(w: Workload, max_num_partitions: Optional[int] = None, fill: f
 
 def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
                  key_cache: Optional[torch.Tensor] = None,
-                 value_cache: Optional[torch.Tensor] = None, timed: bool = True) -> List[float]:
+                 value_cache: Optional[torch.Tensor] = None, timed: bool = True,
+                 max_context_len: Optional[int] = None) -> List[float]:
     """One call of ``lib.paged_attention_<kernel>.run``; returns its kernel times (us).
-    ``key_cache``/``value_cache`` substitute pool clones of the same layout."""
+    ``key_cache``/``value_cache`` substitute pool clones of the same layout.  ``max_context_len``
+    defaults to what the block table can hold (no device read needed to know it)."""
     if kernel.startswith("fp8") != w.is_fp8:
         raise ValueError(f"kernel {kernel} does not match the workload's cache dtype")
     bufs = bufs or alloc_buffers(w)
@@ -60,7 +62,7 @@ def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
     kc = logical_cache_view(w, w.key_cache if key_cache is None else key_cache)
     vc = logical_cache_view(w, w.value_cache if value_cache is None else value_cache)
     G = w.num_heads // w.num_kv_heads
-    max_ctx = int(w.block_tables.shape[1]) * w.block_size
+    max_ctx = max_context_len if max_context_len is not None else int(w.block_tables.shape[1]) * w.block_size
     head = (bufs.max_logits, bufs.exp_sums, bufs.tmp_out, bufs.out, bufs.debug, w.query, kc, vc,
             w.block_tables, w.context_lens, G, w.scale)
     tail = (w.block_size, max_ctx, bufs.alibi, w.sinks, -1.0)

@@ -216,10 +216,11 @@ def test_write_then_attend_with_block_scales(oracle):
         assert err < 0.1, (kernel, float(err))
 
 
-def test_block_scales_in_both_scheduling_forms(oracle):
-    """Per-block scales on a batch the persistent kernels take (100 sequences, several items per
-    work-group) and on one left to the grid form (300 sequences)."""
-    for S, seed in ((100, 71), (300, 72)):
+def test_block_scales_in_every_scheduling_form(oracle):
+    """Per-block scales on a batch the persistent kernels take whole (100 sequences, several items
+    per work-group), on one they take as sub-batches (300 sequences) and on one left to the grid
+    form (a table of 2^24 tokens per sequence)."""
+    for S, seed, wide in ((100, 71, False), (300, 72, False), (7, 73, True)):
         gen = torch.Generator().manual_seed(seed)
         lens = torch.randint(1, 1200, (S,), generator=gen)
         lens[::11] = 0
@@ -227,6 +228,10 @@ def test_block_scales_in_both_scheduling_forms(oracle):
                                fp8=True, block_size=16, seed=seed, fp8_dtype=torch.float8_e4m3fn)
         w.context_lens = lens.to(torch.int32)
         w.partition_size = 256
+        if wide:
+            table = torch.zeros((S, (1 << 24) // w.block_size), dtype=torch.int32)
+            table[:, :w.block_tables.shape[1]] = w.block_tables
+            w.block_tables = table
         NB = w.key_cache.shape[0]
         ks, vs = _scales((NB, 2), seed, 0.2, 3.0), _scales((NB, 2), seed + 1, 0.01, 3.0)
         ref = _ref(oracle, w, k_scales=ks, v_scales=vs)

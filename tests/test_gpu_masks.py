@@ -194,11 +194,12 @@ def test_query_tokens_head_major_e4m3(oracle):
         torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel}: {m}")
 
 
-def test_extended_instances_in_both_scheduling_forms(oracle):
-    """Modifiers + two query tokens on a batch that the persistent kernels take (120 sequences,
-    several items per work-group, empty sequences in between) and on one they leave to the grid
-    form (300 sequences)."""
-    for S, seed in ((120, 31), (300, 32)):
+def test_extended_instances_in_every_scheduling_form(oracle):
+    """Modifiers + two query tokens on a batch that the persistent kernels take whole (120
+    sequences, several items per work-group, empty sequences in between), on one they take as
+    sub-batches (300 sequences) and on one left to the grid form (a table of 2^24 tokens per
+    sequence)."""
+    for S, seed, wide in ((120, 31, False), (300, 32, False), (9, 33, True)):
         gen = torch.Generator().manual_seed(seed)
         lens = torch.randint(1, 1500, (S,), generator=gen)
         lens[::9] = 0
@@ -206,6 +207,10 @@ def test_extended_instances_in_both_scheduling_forms(oracle):
         w = W.make_config(0, num_seqs=S, pool_blocks=S * 94, lens=lens.tolist())     # D 64, G 1
         w.partition_size = 256
         w.sinks = torch.linspace(-2, 2, w.num_heads).to(w.query.dtype)
+        if wide:
+            table = torch.zeros((S, (1 << 24) // w.block_size), dtype=torch.int32)
+            table[:, :w.block_tables.shape[1]] = w.block_tables
+            w.block_tables = table
         H = w.query.shape[1]
         QL = 2
         query4 = torch.randn(S, QL, H, 64, generator=gen).to(torch.float16)

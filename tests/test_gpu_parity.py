@@ -22,11 +22,11 @@ def _dev():
     return torch.device("cuda:0")
 
 
-def _run(w_cpu, kernel, **kw):
+def _run(w_cpu, kernel, max_context_len=None, **kw):
     from flash_attention_factory_amd import runner
     w = w_cpu.to(_dev())
     bufs = runner.alloc_buffers(w, **kw)
-    times = runner.run_workload(w, kernel, bufs)
+    times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len)
     torch.cuda.synchronize()
     return bufs, times
 
@@ -147,9 +147,9 @@ def test_edge_cases(oracle):
     torch.testing.assert_close(out[[1, 3]].float(), ref[[1, 3]].float(), atol=ATOL, rtol=RTOL)
 
 
-def test_large_batch_uses_grid_form_of_split_kernel(oracle):
-    """More than 256 sequences: the split path falls back from the persistent kernel to
-    one work-group per (kv head, partition slot, sequence)."""
+def test_large_batch_runs_as_sub_batches(oracle):
+    """More sequences than the persistent kernels list (256 split, 128 loop): the launchers cut
+    the batch into equal sub-batches, one persistent launch each."""
     gen = torch.Generator().manual_seed(5)
     lens = torch.randint(1, 700, (300,), generator=gen).tolist()
     w = W.make_config(0, num_seqs=300, pool_blocks=300 * 44, lens=lens)
@@ -276,7 +276,7 @@ def test_full_size_configs(oracle, index):
 def test_persistent_kernels_small_batches(oracle):
     """Fewer items than resident work-groups, a single sequence, a batch where most
     wavefronts of a loop work-group have no chunk, and 128 sequences (the limit of the
-    persistent loop kernel) next to 129 (grid form)."""
+    persistent loop kernel) next to 129 (two sub-batches of 65 and 64)."""
     cases = [
         W.make_config(1, num_seqs=1, pool_blocks=200, lens=[1999]),
         W.make_config(0, num_seqs=3, pool_blocks=64, lens=[5, 40, 33]),
@@ -297,8 +297,32 @@ def test_table_wider_than_the_persistent_loop_key(oracle):
     wide = torch.zeros((2, (1 << 24) // w.block_size), dtype=torch.int32)
     wide[:, :w.block_tables.shape[1]] = w.block_tables
     w.block_tables = wide
-    bufs, _ = _run(w, "loop")
-    _check(bufs.out, w, oracle, "2^24-token table/loop")
+    for kernel in ("loop", "reduce"):
+        bufs, _ = _run(w, kernel, max_context_len=40)
+        _check(bufs.out, w, oracle, f"2^24-token table/{kernel}")
+
+
+def test_grid_forms_on_a_ragged_batch(oracle):
+    """The grid forms (one work-group per (kv head[, partition], sequence)) serve what the
+    persistent kernels do not take; a table of 2^24 tokens per sequence selects them.  A ragged
+    batch with sinks, empty sequences and several partitions, 16-bit and E5M2."""
+    gen = torch.Generator().manual_seed(17)
+    lens = torch.randint(1, 1400, (6,), generator=gen)
+    lens[2] = 0
+    for index in (1, 3):
+        w = W.make_config(index, num_seqs=6, pool_blocks=600, lens=lens.tolist())
+        w.sinks = torch.linspace(-1, 1, w.num_heads).to(w.query.dtype)
+        wide = torch.zeros((6, (1 << 24) // w.block_size), dtype=torch.int32)
+        wide[:, :w.block_tables.shape[1]] = w.block_tables
+        w.block_tables = wide
+        for kernel in (("fp8_loop", "fp8_reduce") if w.is_fp8 else ("loop", "reduce")):
+            bufs, _ = _run(w, kernel, max_context_len=int(lens.max()))
+            out = bufs.out.cpu()
+            assert (out[2] == 0).all()
+            ref = call_oracle(oracle.attention_ref, w)
+            live = lens > 0
+            torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL,
+                                       msg=lambda m: f"grid {kernel}: {m}")
 
 
 @pytest.mark.parametrize("qdtype", [torch.float16, torch.bfloat16])
