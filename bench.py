@@ -39,6 +39,9 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (summaries under profiles/); None where not yet measured.
+# 512-sequence variants of the configurations (--large-batches): blocks per pool
+LARGE_BATCH_POOL_BLOCKS = {1: 49152, 3: 49152, 4: 220000}
+
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE + WRITE_SIZE of paged_attn_loop_persistent_kernel<128, F16, kv16> per launch,
     # profiles/paged_attn_kernels_bench_configs.md
@@ -304,6 +307,10 @@ def main():
                     help="other configurations to time besides configuration 1 ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kv-cache-write", action="store_true")
+    ap.add_argument("--large-batches", action="store_true",
+                    help="also time configurations 4, 3 and 1 with 512 sequences (up to 26 GB of pools), "
+                         "each in a process of its own")
+    ap.add_argument("--large-batch-only", type=int, default=-1, help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no multi-GPU form in this build "
@@ -317,6 +324,15 @@ def main():
         return 2
     _cabi.load()  # raises if the HIP library was not built: there is no fallback
     dev = torch.device("cuda:0")
+    if args.large_batch_only >= 0:
+        # a batch beyond what one persistent launch lists: sub-batches (split path, 16-bit loop
+        # path) or the grid form (FP8 loop path)
+        idx = args.large_batch_only
+        big = _build_config(idx, torch, W, runner, dev, num_seqs=512, pool_blocks=LARGE_BATCH_POOL_BLOCKS[idx])
+        _, r = _time_config(big, 20, 3, torch, W, runner, dev)
+        r["workload"] += "_512_sequences"
+        print(json.dumps(r), flush=True)
+        return 0
 
     # All pools are allocated before anything is timed, largest first: memory handed out
     # after other pools were freed is fragmented into small pages, and the randomly
@@ -375,6 +391,20 @@ def main():
         line["kv_cache_write"] = _time_kv_cache_write(max(20, args.steps // 2), torch, dev, not args.no_cpu_baseline)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(1, torch, W)
+    if args.large_batches:
+        # Pools of tens of GB want an allocator nobody has fragmented (see above): one child
+        # process per configuration, after this process has given its own pools back.
+        import subprocess
+        built = None
+        torch.cuda.empty_cache()
+        line["large_batches"] = []
+        for idx in sorted(LARGE_BATCH_POOL_BLOCKS):
+            child = subprocess.run([sys.executable, os.path.abspath(__file__), "--large-batch-only", str(idx)],
+                                   capture_output=True, text=True)
+            if child.returncode != 0:
+                print(child.stderr, file=sys.stderr)
+                return child.returncode
+            line["large_batches"].append(json.loads(child.stdout.strip().splitlines()[-1]))
     print(json.dumps(line), flush=True)
     return 0
 
