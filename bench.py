@@ -16,6 +16,7 @@ cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTor
 configs      the other four configurations, each timed the same way
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
 query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step)
+token_major_layout  configurations 1 and 3 with pools laid out as the reference's tests build them
 kv_block_scales  the FP8 loop configuration with E4M3 pools and per-block K and V scales
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
              the asynchronous torch.library operators, and a HIP-graph replay of them
@@ -384,6 +385,16 @@ def main():
     others.append(r)
     line["kv_block_scales"] = _time_block_scales(e4m3, max(20, args.steps // 2), torch, W, runner, dev)
     del e4m3
+    # configurations 1 and 3 once more with pools in the reference's own layout
+    # [blocks, block_size, kv_heads, head_size]: a token's row of one kv head is then the only
+    # contiguous piece (256 or 128 bytes), successive tokens lie kv_heads rows apart
+    line["token_major_layout"] = []
+    for idx in (1, 3):
+        tm = _build_config(idx, torch, W, runner, dev, layout=W.TOKEN_MAJOR)
+        _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+        r["workload"] += "_token_major"
+        line["token_major_layout"].append(r)
+        del tm
     line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
         del built
