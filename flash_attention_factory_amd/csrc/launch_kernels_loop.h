@@ -33,12 +33,16 @@ inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, cons
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float total_us = 0.f;
-  // One launch per group of query tokens that fit the 16 MFMA columns (one launch for decode).
-  for (int q0 = 0; q0 < r.query_len; q0 += p.query_count) {
+  const bool persistent = kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs &&
+                          shape.num_pool_blocks > 0 && max_ctx < kLoopPersistentMaxContext;
+  // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
+  // columns, or in the persistent form two tiles of 16 held by two halves of every work-group.
+  const int per_tile = p.query_count;
+  const int per_launch = (persistent && r.query_len > per_tile) ? 2 * per_tile : per_tile;
+  for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {
     p.query_first = q0;
-    p.query_count = std::min(p.query_count, r.query_len - q0);
-    if (kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
-        max_ctx < kLoopPersistentMaxContext) {
+    p.query_count = std::min(per_launch, r.query_len - q0);
+    if (persistent) {
       // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
       // sequences first, with the next item's first loads issued before each merge.
       constexpr int PW = PersistentLoop<KV8>::waves;
@@ -46,7 +50,9 @@ inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, cons
                                                      Pipeline<KV8>::tiles_per_chunk, false>;
       auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
                                                         Pipeline<KV8>::tiles_per_chunk, true>;
-      auto kernel = ext ? extended : plain;
+      auto two_tiles = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                         Pipeline<KV8>::tiles_per_chunk, true, 2>;
+      auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
       int resident = 0;
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
       const dim3 grid((unsigned)std::min<int64_t>(resident, items));

@@ -38,25 +38,41 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float attention_us = 0.f;
-  // One launch per group of query tokens that fit the 16 MFMA columns (one launch for decode);
-  // every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
-  for (int q0 = 0; q0 < r.query_len; q0 += p.query_count) {
+  const bool segment_form = SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs &&
+                            shape.num_pool_blocks > 0 &&
+                            (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
+  // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
+  // columns, or in the segment form two tiles of 16 held by two halves of every work-group.
+  // Every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
+  const int per_tile = p.query_count;
+  const int per_launch = (segment_form && r.query_len > per_tile) ? 2 * per_tile : per_tile;
+  for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {
     p.query_first = q0;
-    p.query_count = std::min(p.query_count, r.query_len - q0);
-    if (SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
-        (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext) {
+    p.query_count = std::min(per_launch, r.query_len - q0);
+    if (segment_form) {
       // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
       constexpr int SW = SegmentSplit<KV8>::waves;
       auto plain = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                              Pipeline<KV8>::tiles_per_chunk, false>;
       auto extended = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                                 Pipeline<KV8>::tiles_per_chunk, true>;
-      auto kernel = ext ? extended : plain;
-      int resident = 0;
-      FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
-      const int64_t max_items =
-          (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
-      segment_groups = (int)std::min<int64_t>(resident, max_items);
+      auto two_tiles = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                                 Pipeline<KV8>::tiles_per_chunk, true, 2>;
+      auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
+      if (q0 == 0) {
+        // Every launch of the call gets the same number of work-groups: the segment length, which
+        // the reduce kernel works out again, follows from it.
+        int resident = 0;
+        FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
+        if (ext && r.query_len > per_launch && r.query_len % per_launch <= per_tile) {  // a one-tile launch ends the call
+          int other = 0;
+          FA_HIP_CHECK(resident_groups(extended, SW * 64, &other));
+          resident = std::min(resident, other);
+        }
+        const int64_t max_items =
+            (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
+        segment_groups = (int)std::min<int64_t>(resident, max_items);
+      }
       FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
     } else if (ext) {
       const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);

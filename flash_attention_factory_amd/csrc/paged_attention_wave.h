@@ -124,13 +124,15 @@ struct WaveAttn {
   // EXT: what the normalised output of the item at hand is multiplied with (see ItemExt).
   float out_mul = 1.f;
 
-  __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane)
+  // `tile`: which 16 columns of the launch's (query token, head) pairs this wavefront holds
+  // (kernels with several column tiles per launch; 0 otherwise)
+  __device__ __forceinline__ WaveAttn(const PagedAttnParams &prm, int lane, int tile = 0)
       : p(prm), r(lane >> 4), i(lane & 15), blk_mask((1 << prm.block_shift) - 1) {
     if constexpr (EXT) {
-      const int q = i / prm.group;
-      col_g = i - q * prm.group;
+      const int q = tile * (16 / prm.group) + i / prm.group;  // query token of the launch
+      col_g = i % prm.group;
       col_q = prm.query_first + q;
-      col_valid = q < prm.query_count;
+      col_valid = i < (16 / prm.group) * prm.group && q < prm.query_count;
     } else {
       col_g = i;
       col_valid = i < prm.group;

@@ -144,7 +144,8 @@ typedef struct fa_paged_attention_options {
                                  context (their K/V rows already in the caches, context_lens counting
                                  them) and token j sees the keys up to its own position -- upstream's
                                  causal rule, test_paged.py:79-80.  At most 64.  K and V are read
-                                 once per group of 16 / (num_heads / num_kv_heads) query tokens */
+                                 once per group of 2 * (16 / (num_heads / num_kv_heads)) query
+                                 tokens */
   int32_t kv_scale_mode;      /* FP8 entries and the KV-cache writer: fa_kv_scale.  0 = the scalar
                                  fp8_scale as upstream; otherwise fp8_scale is ignored and the two
                                  arrays below are read */
