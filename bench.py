@@ -46,7 +46,7 @@ LARGE_BATCH_POOL_BLOCKS = {1: 49152, 3: 49152, 4: 220000}
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE + WRITE_SIZE of paged_attn_loop_persistent_kernel<128, F16, kv16> per launch,
     # profiles/paged_attn_kernels_bench_configs.md
-    "config1_loop": 661.22e6 + 0.26e6,
+    "config1_loop": 661.19e6 + 0.26e6,
 }
 
 
@@ -308,6 +308,9 @@ def main():
                     help="other configurations to time besides configuration 1 ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kv-cache-write", action="store_true")
+    ap.add_argument("--no-token-major", action="store_true",
+                    help="skip the token-major legs (they run the same kernels as configurations 1 and 3, "
+                         "which blurs a per-kernel profile)")
     ap.add_argument("--large-batches", action="store_true",
                     help="also time configurations 4, 3 and 1 with 512 sequences (up to 26 GB of pools), "
                          "each in a process of its own")
@@ -389,7 +392,7 @@ def main():
     # [blocks, block_size, kv_heads, head_size]: a token's row of one kv head is then the only
     # contiguous piece (256 or 128 bytes), successive tokens lie kv_heads rows apart
     line["token_major_layout"] = []
-    for idx in (1, 3):
+    for idx in (() if args.no_token_major else (1, 3)):
         tm = _build_config(idx, torch, W, runner, dev, layout=W.TOKEN_MAJOR)
         _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
         r["workload"] += "_token_major"
