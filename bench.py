@@ -15,7 +15,8 @@ cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTor
              reference) on the same workload on this box's host cores
 configs      the other four configurations, each timed the same way
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
-query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step)
+query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step);
+             query_tokens_two_tiles: with 32, which fill two tiles of MFMA columns
 token_major_layout  configurations 1 and 3 with pools laid out as the reference's tests build them
 kv_block_scales  the FP8 loop configuration with E4M3 pools and per-block K and V scales
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
@@ -381,6 +382,9 @@ def main():
     }
     line["score_modifiers"] = _time_score_modifiers(built[1], max(20, args.steps // 2), torch, W, runner, dev)
     line["query_tokens"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev)
+    # 32 tokens of one head are two column tiles, held by two halves of every work-group
+    line["query_tokens_two_tiles"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev,
+                                                        query_len=32)
     # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
     e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
     _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
