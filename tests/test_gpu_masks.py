@@ -251,3 +251,30 @@ def test_more_query_tokens_than_the_mfma_columns_hold(oracle, QL, nheads, nheads
                           window_left=300).float().cpu()
         assert torch.isfinite(got).all(), kernel
         torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel} QL={QL}: {m}")
+
+
+@pytest.mark.parametrize("index,QL", [(4, 4), (1, 32), (2, 8)])
+def test_full_size_query_blocks_with_modifiers(oracle, index, QL):
+    """The measured configurations at full size with a query block of two column tiles (G x QL =
+    32 columns), a local window and ALiBi, through the loop and the split entry: whole output
+    against the oracle, and loop == split within two 16-bit roundings."""
+    dev = _dev()
+    wd = W.make_config(index, device=dev, pools_on_device=True)
+    w = wd.to("cpu")
+    S, H, D = w.query.shape
+    g = torch.Generator().manual_seed(40 + index)
+    query4 = torch.randn(S, QL, H, D, generator=g).to(w.query.dtype)
+    alibi = torch.linspace(0.0005, 0.01, H)
+    window = int(w.context_lens.max()) // 2
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               fp8_scale=w.fp8_scale, want_f32=True, alibi_slopes=alibi, window_left=window)[1]
+    outs = {}
+    for kernel in (("fp8_loop", "fp8_reduce") if w.is_fp8 else ("loop", "reduce")):
+        got = _call_multi(wd, query4.to(dev), kernel, alibi_slopes=alibi.to(dev), apply_alibi=True,
+                          window_left=window).float().cpu()
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"config {index} {kernel}: {m}")
+        outs[kernel] = got
+    a, b = outs.values()
+    ulps = 2.0 ** (-7 if w.query.dtype == torch.bfloat16 else -10)
+    assert (a - b).abs().max().item() <= ulps * ref.abs().max().item() + 1e-5
