@@ -20,11 +20,13 @@
  * last failure on the calling thread is available from fa_last_error().
  *
  * Tensor shapes (row-major, innermost dimension contiguous):
- *   out, query      [num_seqs, num_heads, head_size]            q_dtype (fp16 / bf16)
+ *   out, query      [num_seqs, num_heads, head_size]            q_dtype (fp16 / bf16);
+ *                   [num_seqs, query_len, num_heads, head_size] with options->query_len > 1
  *   key_cache,      a pool of blocks addressed with explicit element strides
  *   value_cache       element(block b, token t, kv head h, dim d) =
  *                       base[b*kv_block_stride + t*kv_token_stride + h*kv_head_stride + d]
- *                     16-bit caches hold q_dtype values, FP8 caches hold E5M2 bytes.
+ *                     16-bit caches hold q_dtype values, FP8 caches hold E5M2 bytes (as
+ *                     upstream) or E4M3 bytes (options->kv_fp8_format).
  *                     upstream layout [blocks, block_size, kv_heads, head_size]
  *                       -> strides (block_size*kv_heads*head_size, kv_heads*head_size, head_size)
  *                     head-major layout [blocks, kv_heads, block_size, head_size]
@@ -153,7 +155,8 @@ typedef struct fa_paged_attention_options {
   const float *v_scales;
 } fa_paged_attention_options;
 
-/* Single-pass kernel: one launch, no scratch. */
+/* Single-pass kernel: no scratch.  One launch for a decode batch of up to 128 sequences; larger
+ * batches and query blocks of more than 32 (token, head) columns per kv head take several. */
 int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_cache,
                                 const void *value_cache, const int32_t *block_tables,
                                 const int32_t *context_lens, float scale, int32_t max_context_len,
@@ -172,7 +175,7 @@ int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_
                                   float *tmp_out, const fa_paged_attention_shape *shape,
                                   const fa_paged_attention_options *options);
 
-/* FP8-E5M2 KV-cache variants: caches are bytes, dequantised in registers. */
+/* FP8 KV-cache variants: caches are bytes (E5M2 as upstream, or E4M3), dequantised in registers. */
 int32_t fa_paged_attention_fp8_loop(void *out, const void *query, const void *key_cache,
                                     const void *value_cache, const int32_t *block_tables,
                                     const int32_t *context_lens, float scale,
