@@ -153,9 +153,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   if (o && o->query_len < 0) return fail(FA_ERR_BAD_SHAPE, "query_len must be >= 0");
   if (r->query_len > kMaxQueryLen)
     return fail(FA_ERR_BAD_SHAPE, "query_len %d exceeds %d", r->query_len, kMaxQueryLen);
-  if ((int64_t)s->num_seqs * r->query_len > 65535)
-    return fail(FA_ERR_BAD_SHAPE, "num_seqs x query_len %lld exceeds the grid limit 65535",
-                (long long)s->num_seqs * r->query_len);
+  if ((int64_t)s->num_seqs * r->query_len * s->num_heads > 0x7fffffffLL)
+    return fail(FA_ERR_BAD_SHAPE, "num_seqs x query_len x num_heads %lld exceeds the grid limit 2^31 - 1",
+                (long long)s->num_seqs * r->query_len * s->num_heads);
   r->alibi_slopes = o ? o->alibi_slopes : nullptr;
   r->softcap = o ? o->softcap : 0.f;
   r->window_left = o ? o->window_left : 0;

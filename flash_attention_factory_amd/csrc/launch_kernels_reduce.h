@@ -105,7 +105,7 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   rp.num_kv_heads = shape.num_kv_heads;
   rp.query_len = r.query_len;
   rp.segment_groups = segment_groups;
-  const dim3 rgrid(shape.num_heads, shape.num_seqs * r.query_len);
+  const dim3 rgrid((unsigned)((int64_t)shape.num_heads * shape.num_seqs * r.query_len));
   const bool one_wave = (int64_t)shape.num_heads * shape.num_seqs * r.query_len >= kReduceSingleWaveMinPairs;
   if (segment_groups > 0) {
     if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, true>, rgrid, dim3(64), 1, rp));

@@ -57,8 +57,10 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   constexpr int R = reduce_rows_in_flight<SEGMENTS>();
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int head = blockIdx.x;
-  const int seq = blockIdx.y;  // row of out and of the scratch arrays
+  // one work-group per (row, head), heads fastest; a row of out and of the scratch arrays is a
+  // sequence, or a (sequence, query token) pair
+  const int seq = blockIdx.x / p.num_heads;
+  const int head = blockIdx.x - seq * p.num_heads;
   const int ctx = min(p.context_lens[p.query_len > 1 ? seq / p.query_len : seq], p.max_context);
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;

@@ -278,3 +278,21 @@ def test_full_size_query_blocks_with_modifiers(oracle, index, QL):
     a, b = outs.values()
     ulps = 2.0 ** (-7 if w.query.dtype == torch.bfloat16 else -10)
     assert (a - b).abs().max().item() <= ulps * ref.abs().max().item() + 1e-5
+
+
+def test_more_rows_than_one_grid_dimension_holds(oracle):
+    """2100 sequences x 32 query tokens = 67200 rows of out and scratch: more than the 65535 a
+    second grid dimension could address; both entry points, tiny contexts."""
+    S, QL = 2100, 32
+    gen = torch.Generator().manual_seed(77)
+    lens = torch.randint(1, 40, (S,), generator=gen)
+    w = W.make_config(0, num_seqs=S, pool_blocks=S * 3, lens=lens.tolist())      # D 64, G 1, 8 heads
+    H = w.query.shape[1]
+    query4 = torch.randn(S, QL, H, 64, generator=gen).to(torch.float16)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               want_f32=True)[1]
+    wd = w.to(_dev())
+    for kernel in ("loop", "reduce"):
+        got = _call_multi(wd, query4.to(_dev()), kernel).float().cpu()
+        torch.testing.assert_close(got, ref, atol=ATOL, rtol=RTOL, msg=lambda m: f"{kernel}: {m}")
