@@ -5,6 +5,7 @@ as the benchmark contract states; the upstream relative rule
 in the form err <= 3 * err(oracle kernel model) + 1e-5 where the kernel model rounds
 where the upstream kernels round."""
 import math
+import os
 
 import pytest
 import torch
@@ -379,3 +380,42 @@ def test_bf16_and_fp8_scale(oracle):
     for kernel in ("fp8_loop", "fp8_reduce"):
         bufs, _ = _run(w8, kernel)
         _check(bufs.out, w8, oracle, f"bf16 q, fp8 cache, scale 0.5/{kernel}")
+
+
+UPSTREAM_HEADS = [(8, 1), (16, 2), (10, 2), (14, 2), (12, 2), (8, 2), (6, 2), (4, 2), (2, 2)]
+UPSTREAM_SHORT = [128, 339, 1024, 800, 256, 799, 2048]
+UPSTREAM_LONG = [20000, 40000, 50000]
+
+
+@pytest.mark.parametrize("heads", UPSTREAM_HEADS, ids=lambda h: f"h{h[0]}x{h[1]}")
+@pytest.mark.parametrize("fp8", [False, True])
+def test_whole_upstream_grid(oracle, heads, fp8):
+    """Every case of the upstream test grid (test_paged.py:211-256, test_paged_fp8cache.py:220-264:
+    batch 1/2 x sinks x var-len x head size 128/64 x nine head pairs x ten context lengths, block
+    64, fp16) through the loop and the split kernel, with upstream's own gate next to the
+    absolute one (err <= 3 x err of the rounding-faithful model + 1e-5, test_paged.py:603-604).
+    The seven lengths up to 2048 in full; of the three long ones (20000-50000) one combination of
+    the other parameters each, rotating -- the oracle needs a third of a second for those -- unless
+    FA_FULL_UPSTREAM_GRID=1 asks for all 2 x 1440 cases."""
+    nheads, nheads_k = heads
+    combos = [(b, s, v, d) for b in (1, 2) for s in (True, False) for v in (False, True) for d in (128, 64)]
+    n = 0
+    for seqlen_k in UPSTREAM_SHORT:
+        for b, s, v, d in combos:
+            w = W.make_test_shaped(batch_size=b, nheads=nheads, nheads_k=nheads_k, d=d, seqlen_k=seqlen_k, varlen=v,
+                                   has_sinks=s, fp8=fp8)
+            for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+                bufs, _ = _run(w, kernel)
+                _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
+            n += 1
+    everything = os.environ.get("FA_FULL_UPSTREAM_GRID") == "1"   # the long lengths in full too: minutes
+    for k, seqlen_k in enumerate(UPSTREAM_LONG):
+        one = combos[(3 * UPSTREAM_HEADS.index(heads) + k + (8 if fp8 else 0)) % len(combos)]
+        for b, s, v, d in (combos if everything else [one]):
+            w = W.make_test_shaped(batch_size=b, nheads=nheads, nheads_k=nheads_k, d=d, seqlen_k=seqlen_k, varlen=v,
+                                   has_sinks=s, fp8=fp8)
+            for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+                bufs, _ = _run(w, kernel)
+                _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
+            n += 1
+    assert n == len(UPSTREAM_SHORT) * 16 + len(UPSTREAM_LONG) * (16 if everything else 1)
