@@ -74,31 +74,16 @@ __device__ __forceinline__ float load_scalar16<BF16>(const void *p) {
   return (float)*reinterpret_cast<const __bf16 *>(p);
 }
 
-// E5M2 is binary16 cut to its top byte: byte b decodes to the fp16 with bits b << 8.
-// e5m2_pair<QT>(lo_byte, hi_byte) builds one dword holding the two decoded values in
-// the query dtype.  Bytes arrive already isolated in bits 0..7.
-template <typename QT>
-__device__ __forceinline__ uint32_t e5m2_pair(uint32_t lo_byte, uint32_t hi_byte);
-template <>
-__device__ __forceinline__ uint32_t e5m2_pair<F16>(uint32_t lo_byte, uint32_t hi_byte) {
-  return (lo_byte << 8) | (hi_byte << 24);
-}
-template <>
-__device__ __forceinline__ uint32_t e5m2_pair<BF16>(uint32_t lo_byte, uint32_t hi_byte) {
-  // v_cvt_scalef32_pk_bf16_bf8 decodes bytes 0 and 1 of its source; E5M2 -> bf16 is
-  // exact (2 mantissa bits, exponent range inside bf16's).
-  uint32_t two = lo_byte | (hi_byte << 8);
-  bf16x2 v = __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(two, 1.0f, false);
-  return __builtin_bit_cast(uint32_t, v);
-}
-
+// E5M2 is binary16 cut to its top byte: byte b decodes to the fp16 with bits b << 8; into bf16
+// it goes through v_cvt_scalef32_pk_bf16_bf8 (exact: 2 mantissa bits, exponent range inside
+// bf16's).
 // Dword w holds four E5M2 bytes; decode bytes (2*half, 2*half+1) to a 16-bit pair.
 template <typename QT>
 __device__ __forceinline__ uint32_t e5m2_adjacent_pair(uint32_t w, int half);
 template <>
 __device__ __forceinline__ uint32_t e5m2_adjacent_pair<F16>(uint32_t w, int half) {
-  return half == 0 ? (((w & 0xffu) << 8) | ((w & 0xff00u) << 16))
-                   : (((w >> 8) & 0xff00u) | (w & 0xff000000u));
+  // one byte permute: result bytes (0, w[2*half], 0, w[2*half + 1]); selector 0x0c yields zero
+  return half == 0 ? __builtin_amdgcn_perm(w, w, 0x010c000cu) : __builtin_amdgcn_perm(w, w, 0x030c020cu);
 }
 template <>
 __device__ __forceinline__ uint32_t e5m2_adjacent_pair<BF16>(uint32_t w, int half) {
@@ -112,17 +97,26 @@ __device__ __forceinline__ uint32_t e5m2_adjacent_pair<BF16>(uint32_t w, int hal
 // both decode exactly into fp16 and bf16.
 constexpr int kKv16 = 0, kKvE5M2 = 1, kKvE4M3 = 2;
 
+// Decode byte k (0..3) of dword y into the low and byte k of dword x into the high 16-bit
+// half: the V transpose takes its two tokens from two registers.  One byte permute does the
+// gather -- for E5M2 into fp16 it is the whole decode (bytes land in the top halves), otherwise
+// it puts the bytes next to each other for the conversion instruction.
 template <int KVF, typename QT>
-__device__ __forceinline__ uint32_t fp8_pair(uint32_t lo_byte, uint32_t hi_byte) {
-  if constexpr (KVF == kKvE4M3) {
-    const uint32_t two = lo_byte | (hi_byte << 8);
-    if constexpr (std::is_same<QT, BF16>::value) {
-      return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(two, 1.0f, false));
-    } else {
-      return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(two, 1.0f, false));
-    }
+__device__ __forceinline__ uint32_t fp8_pair_at(uint32_t y, uint32_t x, int k) {
+  // v_perm_b32 selectors: 0..3 = bytes of the second operand, 4..7 = bytes of the first, 0x0c = 0
+  if constexpr (KVF == kKvE5M2 && std::is_same<QT, F16>::value) {
+    return __builtin_amdgcn_perm(x, y, 0x000c000cu | ((uint32_t)k << 8) | ((uint32_t)(4 + k) << 24));
   } else {
-    return e5m2_pair<QT>(lo_byte, hi_byte);
+    const uint32_t two = __builtin_amdgcn_perm(x, y, 0x0c0c0000u | (uint32_t)k | ((uint32_t)(4 + k) << 8));
+    if constexpr (KVF == kKvE4M3) {
+      if constexpr (std::is_same<QT, BF16>::value) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(two, 1.0f, false));
+      } else {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(two, 1.0f, false));
+      }
+    } else {
+      return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(two, 1.0f, false));
+    }
   }
 }
 template <int KVF, typename QT>

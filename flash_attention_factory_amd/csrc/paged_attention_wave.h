@@ -311,9 +311,7 @@ struct WaveAttn {
         const uint32_t y = R.v[e0][dt >> 1], x = R.v[e0 + 1][dt >> 1];
         o[c] = (dt & 1) ? ((y >> 16) | (x & 0xffff0000u)) : ((y & 0xffffu) | (x << 16));
       } else {
-        const uint32_t y = (R.v[e0][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
-        const uint32_t x = (R.v[e0 + 1][dt >> 2] >> (8 * (dt & 3))) & 0xffu;
-        o[c] = fp8_pair<KVF, QT>(y, x);
+        o[c] = fp8_pair_at<KVF, QT>(R.v[e0][dt >> 2], R.v[e0 + 1][dt >> 2], dt & 3);
       }
     }
     return o;
