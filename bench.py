@@ -47,7 +47,7 @@ LARGE_BATCH_POOL_BLOCKS = {1: 49152, 3: 49152, 4: 220000}
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE + WRITE_SIZE of paged_attn_loop_persistent_kernel<128, F16, kv16> per launch,
     # profiles/paged_attn_kernels_bench_configs.md
-    "config1_loop": 661.19e6 + 0.26e6,
+    "config1_loop": 661.20e6 + 0.26e6,
 }
 
 
