@@ -19,6 +19,10 @@ FA_ERR_UNSUPPORTED_DTYPE = 4
 FA_ERR_PARTITION_OVERFLOW = 5
 FA_ERR_BAD_SHAPE = 6
 FA_ERR_RUNTIME = 7
+FA_ERR_SCRATCH_TOO_SMALL = 8
+
+# bytes of the library-owned scratch of fa_paged_attention_reduce_static_scratch
+FA_STATIC_SCRATCH_BYTES = 64 << 20
 
 FA_DTYPE_F16 = 0
 FA_DTYPE_BF16 = 1
@@ -31,6 +35,7 @@ EXPORTS = (
     "fa_last_error",
     "fa_paged_attention_abi_version",
     "fa_kv_cache_write",
+    "fa_paged_attention_reduce_static_scratch",
 )
 
 FA_KV_CACHE_16BIT = 0
@@ -148,7 +153,7 @@ def load() -> ctypes.CDLL:
     P = ctypes.c_void_p
     common = [P, P, P, P, P, P, ctypes.c_float, ctypes.c_int32]
     tail = [ctypes.POINTER(Shape), ctypes.POINTER(Options)]
-    for name in ("fa_paged_attention_loop", "fa_paged_attention_fp8_loop"):
+    for name in ("fa_paged_attention_loop", "fa_paged_attention_fp8_loop", "fa_paged_attention_reduce_static_scratch"):
         fn = getattr(L, name)
         fn.argtypes = common + tail
         fn.restype = ctypes.c_int32

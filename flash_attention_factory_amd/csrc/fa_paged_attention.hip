@@ -1,6 +1,8 @@
 // extern "C" surface of libfa_paged_attention.so: four decode entry points, one per host
 // launcher, declared in include/fa_paged_attention.h, and the KV-cache writer declared in
 // include/fa_kv_cache.h.
+#include <mutex>
+
 #include "../../include/fa_kv_cache.h"
 #include "../../include/fa_paged_attention.h"
 
@@ -32,6 +34,76 @@ FA_EXPORT int32_t fa_paged_attention_reduce(void *out, const void *query, const 
   return fa::dispatch_paged_attention(out, query, key_cache, value_cache, block_tables,
                                       context_lens, scale, max_context_len, exp_sums, max_logits,
                                       tmp_out, shape, options);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------
+// Scratch of the split path (exp_sums, max_logits, tmp_out) in a fixed device array.  In host
+// code the name `scratch` is only a handle for hipGetSymbolAddress: each GPU holds its own copy
+// of the array at its own address, asked for once per device and kept in scratch_address.
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kScratchMaxDevices = 64;
+std::mutex scratch_mutex;
+void *scratch_address[kScratchMaxDevices];  // nullptr until the device's first call
+
+// Device address of `scratch` on the current device.
+fa_status static_scratch_of_current_device(unsigned char **base) {
+  int dev = 0;
+  FA_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kScratchMaxDevices)
+    return fa::fail(FA_ERR_RUNTIME, "device %d is beyond the %d devices the static scratch serves", dev,
+                    kScratchMaxDevices);
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (scratch_address[dev] == nullptr) {
+    void *address = nullptr;
+    FA_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+    if (address == nullptr) return fa::fail(FA_ERR_RUNTIME, "hipGetSymbolAddress gave no address for the static scratch");
+    scratch_address[dev] = address;
+  }
+  *base = static_cast<unsigned char *>(scratch_address[dev]);
+  return FA_OK;
+}
+
+}  // namespace
+
+FA_EXPORT int32_t fa_paged_attention_reduce_static_scratch(void *out, const void *query, const void *key_cache,
+                                                           const void *value_cache, const int32_t *block_tables,
+                                                           const int32_t *context_lens, float scale,
+                                                           int32_t max_context_len,
+                                                           const fa_paged_attention_shape *shape,
+                                                           const fa_paged_attention_options *options) {
+  fa::error_buffer()[0] = 0;
+  if (!shape) return fa::fail(FA_ERR_NULL_POINTER, "shape is NULL");
+  if (options && options->elapsed_us)
+    return fa::fail(FA_ERR_BAD_SHAPE, "fa_paged_attention_reduce_static_scratch allocates nothing, events included: "
+                                      "elapsed_us must be NULL (time the call with fa_paged_attention_reduce)");
+  if (shape->num_seqs <= 0 || shape->num_heads <= 0 || shape->max_num_partitions <= 0 || shape->head_size <= 0)
+    return fa::fail(FA_ERR_BAD_SHAPE, "num_seqs, num_heads, max_num_partitions and head_size must be positive");
+  const int64_t query_len = (options && options->query_len > 1) ? options->query_len : 1;
+  const int64_t slots = (int64_t)shape->num_seqs * query_len * shape->num_heads * shape->max_num_partitions;
+  const int64_t scalars = (slots * 4 + 255) / 256 * 256;  // bytes of exp_sums, and of max_logits
+  const int64_t need = 2 * scalars + slots * shape->head_size * 4;
+  if (need > (int64_t)FA_STATIC_SCRATCH_BYTES)
+    return fa::fail(FA_ERR_SCRATCH_TOO_SMALL,
+                    "%lld scratch slots of head size %d need %lld bytes, the static scratch holds %lld: "
+                    "lower max_num_partitions or use fa_paged_attention_reduce with scratch of your own",
+                    (long long)slots, shape->head_size, (long long)need, (long long)FA_STATIC_SCRATCH_BYTES);
+  // validate_only launches nothing and must work without a GPU: any non-NULL aligned address will do
+  static float placeholder[4] __attribute__((aligned(16)));
+  unsigned char *base = reinterpret_cast<unsigned char *>(placeholder);
+  int64_t off_ml = 0, off_tmp = 0;
+  if (!(options && options->validate_only)) {
+    const fa_status st = static_scratch_of_current_device(&base);
+    if (st != FA_OK) return st;
+    off_ml = scalars;
+    off_tmp = 2 * scalars;
+  }
+  return fa::dispatch_paged_attention(out, query, key_cache, value_cache, block_tables, context_lens, scale,
+                                      max_context_len, reinterpret_cast<float *>(base),
+                                      reinterpret_cast<float *>(base + off_ml),
+                                      reinterpret_cast<float *>(base + off_tmp), shape, options);
 }
 
 FA_EXPORT int32_t fa_paged_attention_fp8_loop(void *out, const void *query, const void *key_cache,
@@ -68,4 +140,4 @@ FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *ke
 
 FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
 
-FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 5; }
+FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 6; }

@@ -43,7 +43,11 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
              max_context_len: int, alibi_slopes, sinks: Optional[torch.Tensor], softcap: float,
              partition_size: int = 0, timed: bool = True, apply_alibi: bool = False,
              apply_softcap: bool = False, window_left: Optional[int] = None,
-             k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None) -> List[float]:
+             k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None,
+             static_scratch_partitions: int = 0) -> List[float]:
+    """``static_scratch_partitions`` > 0 (split entries without FP8 only): the scratch arrays are the
+    library's own fixed device array instead of max_logits / exp_sums / tem_output, which may then be
+    None; the value is max_num_partitions."""
     L = _cabi.load()
     if not query.is_cuda:
         raise RuntimeError("paged attention runs on the GPU only: `query` is not a device tensor")
@@ -77,7 +81,7 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     sh.num_kv_heads = key_cache.size(2)
     sh.block_size = block_size
     sh.max_blocks_per_seq = block_tables.size(1)
-    sh.max_num_partitions = max_logits.size(-1) if split else 1
+    sh.max_num_partitions = (static_scratch_partitions or max_logits.size(-1)) if split else 1
     sh.partition_size = partition_size
     sh.kv_block_stride, sh.kv_token_stride, sh.kv_head_stride = (
         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
@@ -118,7 +122,9 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     fn = getattr(L, entry)
     args = [output.data_ptr(), query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
             block_tables.data_ptr(), context_lens.data_ptr(), float(sm_scale), int(max_context_len)]
-    if split:
+    if split and static_scratch_partitions:
+        pass  # the entry point brings its own scratch
+    elif split:
         tmp = _fp32_scratch(tem_output, (S * QL, H, sh.max_num_partitions, D))
         if max_logits.numel() != S * QL * H * sh.max_num_partitions or exp_sums.numel() != max_logits.numel():
             raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,

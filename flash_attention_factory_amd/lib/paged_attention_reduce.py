@@ -18,3 +18,15 @@ def run(max_logits, exp_sums, tem_output, output, debug_output, query, key_cache
                     num_queries_per_tokens, sm_scale, 1.0, block_size, max_context_len,
                     alibi_slopes, sinks, softcap, timed=timed, partition_size=partition_size, apply_alibi=apply_alibi,
                     apply_softcap=apply_softcap, window_left=window_left)
+
+
+def run_static_scratch(output, query, key_cache, value_cache, block_tables, context_lens, num_queries_per_tokens,
+                       sm_scale, block_size, max_context_len, max_num_partitions, sinks=None, *, partition_size=0):
+    """``run`` for callers that cannot allocate (no upstream counterpart): the C entry point
+    ``fa_paged_attention_reduce_static_scratch`` keeps max_logits, exp_sums and tem_output in a fixed
+    device array of the library (``_cabi.FA_STATIC_SCRATCH_BYTES``), allocates nothing and is always
+    asynchronous on the current stream.  Calls that may overlap on one GPU race for that array."""
+    return run_impl("fa_paged_attention_reduce_static_scratch", True, False, None, None, None, output, None, query,
+                    key_cache, value_cache, block_tables, context_lens, num_queries_per_tokens, sm_scale, 1.0,
+                    block_size, max_context_len, None, sinks, 0.0, timed=False, partition_size=partition_size,
+                    static_scratch_partitions=max_num_partitions)

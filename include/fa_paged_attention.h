@@ -70,7 +70,9 @@ typedef enum fa_status {
   FA_ERR_UNSUPPORTED_DTYPE = 4,
   FA_ERR_PARTITION_OVERFLOW = 5, /* max_context_len needs more than max_num_partitions */
   FA_ERR_BAD_SHAPE = 6,          /* non-positive sizes, misaligned strides or pointers */
-  FA_ERR_RUNTIME = 7             /* a HIP call failed; see fa_last_error() */
+  FA_ERR_RUNTIME = 7,            /* a HIP call failed; see fa_last_error() */
+  FA_ERR_SCRATCH_TOO_SMALL = 8   /* fa_paged_attention_reduce_static_scratch: the call needs more
+                                    scratch than FA_STATIC_SCRATCH_BYTES */
 } fa_status;
 
 typedef enum fa_dtype { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 } fa_dtype;
@@ -174,6 +176,29 @@ int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_
                                   int32_t max_context_len, float *exp_sums, float *max_logits,
                                   float *tmp_out, const fa_paged_attention_shape *shape,
                                   const fa_paged_attention_options *options);
+
+/* fa_paged_attention_reduce for callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart upstream (there
+ * the caller allocates max_logits, exp_sums and tem_output, test_paged.py:449-457).  Same kernels,
+ * same arguments and same `out` as fa_paged_attention_reduce, but exp_sums, max_logits and tmp_out
+ * live in a fixed array of FA_STATIC_SCRATCH_BYTES that the library holds in device memory on
+ * every GPU it runs on until the process ends.  The call allocates nothing, on the host or on the
+ * device, and frees nothing.
+ *   needs  2 * align256(4 * slots) + 4 * slots * head_size bytes,
+ *          slots = num_seqs * max(query_len, 1) * num_heads * max_num_partitions;
+ *          more than FA_STATIC_SCRATCH_BYTES -> FA_ERR_SCRATCH_TOO_SMALL, nothing is launched
+ *   options->elapsed_us must be NULL (timing creates events): the call is always asynchronous
+ * Every call a process makes on a GPU uses that GPU's one array and finds the last call's
+ * contents in it: calls whose kernels may overlap on one GPU (two streams, two threads) race --
+ * order them on one stream or with events.  Nothing in the array has to start at zero: every
+ * slot the reduce kernel reads was written by the attention kernel of the same call. */
+#define FA_STATIC_SCRATCH_BYTES (64u << 20)
+int32_t fa_paged_attention_reduce_static_scratch(void *out, const void *query, const void *key_cache,
+                                                 const void *value_cache, const int32_t *block_tables,
+                                                 const int32_t *context_lens, float scale,
+                                                 int32_t max_context_len,
+                                                 const fa_paged_attention_shape *shape,
+                                                 const fa_paged_attention_options *options);
 
 /* FP8 KV-cache variants: caches are bytes (E5M2 as upstream, or E4M3), dequantised in registers. */
 int32_t fa_paged_attention_fp8_loop(void *out, const void *query, const void *key_cache,

@@ -29,7 +29,7 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 5
+    assert L.fa_paged_attention_abi_version() == 6
 
 
 def test_struct_layouts_match_header():
@@ -216,3 +216,23 @@ def test_kv_scale_argument_checks(L):
     assert _kv_write(L, scale_mode=BLOCK, k_scales=0x1000)[0] == _cabi.FA_ERR_NULL_POINTER
     assert _kv_write(L, scale_mode=9, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _kv_write(L, scale_mode=9, cache_dtype=_cabi.FA_KV_CACHE_16BIT)[0] == _cabi.FA_OK
+
+
+def test_static_scratch_rejects_what_does_not_fit(L):
+    # the entry point that allocates nothing: a fixed array holds its scratch, so sizes have a limit
+    sh = _cabi.Shape()
+    for k, v in dict(num_seqs=64, num_heads=64, num_kv_heads=8, head_size=128, block_size=16, max_blocks_per_seq=2048,
+                     max_num_partitions=64, partition_size=0, kv_block_stride=8 * 16 * 128, kv_token_stride=128,
+                     kv_head_stride=16 * 128, q_dtype=_cabi.FA_DTYPE_F16, num_pool_blocks=1 << 16).items():
+        setattr(sh, k, v)
+    op = _cabi.Options()
+    op.validate_only = 1
+    p = 0x1000
+    rc = L.fa_paged_attention_reduce_static_scratch(p, p, p, p, p, p, 0.1, 0, ctypes.byref(sh), ctypes.byref(op))
+    assert rc == _cabi.FA_ERR_SCRATCH_TOO_SMALL and b"static scratch holds" in L.fa_last_error()
+    sh.num_seqs = 8  # 8 * 64 * 64 slots x 130 floats = 17 MB: fits
+    assert L.fa_paged_attention_reduce_static_scratch(p, p, p, p, p, p, 0.1, 0, ctypes.byref(sh), ctypes.byref(op)) == 0
+    elapsed = (ctypes.c_float * 2)()
+    op.elapsed_us = ctypes.cast(elapsed, ctypes.POINTER(ctypes.c_float))
+    rc = L.fa_paged_attention_reduce_static_scratch(p, p, p, p, p, p, 0.1, 0, ctypes.byref(sh), ctypes.byref(op))
+    assert rc == _cabi.FA_ERR_BAD_SHAPE and b"elapsed_us must be NULL" in L.fa_last_error()
