@@ -312,6 +312,11 @@ def main():
     ap.add_argument("--no-token-major", action="store_true",
                     help="skip the token-major legs (they run the same kernels as configurations 1 and 3, "
                          "which blurs a per-kernel profile)")
+    ap.add_argument("--layout", choices=["head_major", "token_major"], default="head_major",
+                    help="pool layout of the main configurations (token_major = the reference's own "
+                         "[blocks, block_size, kv_heads, head_size]); for profiling one layout alone")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="time the configurations only: no modifier, query-token, E4M3, scale or stream-ordered legs")
     ap.add_argument("--large-batches", action="store_true",
                     help="also time configurations 4, 3 and 1 with 512 sequences (up to 26 GB of pools), "
                          "each in a process of its own")
@@ -344,7 +349,7 @@ def main():
     # addressed KV blocks then pay TLB misses that have nothing to do with the kernels.
     indices = [1] + [int(x) for x in args.configs.split(",") if x.strip() != ""]
     order = sorted(set(indices), key=lambda i: -W._CONFIGS[i]["NB"] * W._CONFIGS[i]["Hk"])
-    built = {i: _build_config(i, torch, W, runner, dev) for i in order}
+    built = {i: _build_config(i, torch, W, runner, dev, layout=args.layout) for i in order}
     torch.cuda.synchronize()
 
     _, main_res = _time_config(built[1], args.steps, args.warmup, torch, W, runner, dev)
@@ -380,29 +385,30 @@ def main():
                      "kernel_us": kernel_us},
         "configs": others,
     }
-    line["score_modifiers"] = _time_score_modifiers(built[1], max(20, args.steps // 2), torch, W, runner, dev)
-    line["query_tokens"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev)
-    # 32 tokens of one head are two column tiles, held by two halves of every work-group
-    line["query_tokens_two_tiles"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev,
-                                                        query_len=32)
-    # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
-    e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
-    _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
-    r["workload"] += "_e4m3"
-    others.append(r)
-    line["kv_block_scales"] = _time_block_scales(e4m3, max(20, args.steps // 2), torch, W, runner, dev)
-    del e4m3
-    # configurations 1 and 3 once more with pools in the reference's own layout
-    # [blocks, block_size, kv_heads, head_size]: a token's row of one kv head is then the only
-    # contiguous piece (256 or 128 bytes), successive tokens lie kv_heads rows apart
-    line["token_major_layout"] = []
-    for idx in (() if args.no_token_major else (1, 3)):
-        tm = _build_config(idx, torch, W, runner, dev, layout=W.TOKEN_MAJOR)
-        _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
-        r["workload"] += "_token_major"
-        line["token_major_layout"].append(r)
-        del tm
-    line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
+    if not args.no_extras:
+        line["score_modifiers"] = _time_score_modifiers(built[1], max(20, args.steps // 2), torch, W, runner, dev)
+        line["query_tokens"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev)
+        # 32 tokens of one head are two column tiles, held by two halves of every work-group
+        line["query_tokens_two_tiles"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev,
+                                                            query_len=32)
+        # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
+        e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
+        _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+        r["workload"] += "_e4m3"
+        others.append(r)
+        line["kv_block_scales"] = _time_block_scales(e4m3, max(20, args.steps // 2), torch, W, runner, dev)
+        del e4m3
+        # configurations 1 and 3 once more with pools in the reference's own layout
+        # [blocks, block_size, kv_heads, head_size]: a token's row of one kv head is then the only
+        # contiguous piece (256 or 128 bytes), successive tokens lie kv_heads rows apart
+        line["token_major_layout"] = []
+        for idx in (() if args.no_token_major else (1, 3)):
+            tm = _build_config(idx, torch, W, runner, dev, layout=W.TOKEN_MAJOR)
+            _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+            r["workload"] += "_token_major"
+            line["token_major_layout"].append(r)
+            del tm
+        line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
         del built
         torch.cuda.empty_cache()

@@ -22,6 +22,12 @@
 #include "paged_attention_policy.h"
 #include "paged_attention_utils.h"
 
+// K tiles with rows of 128 bytes or more are loaded a whole 128-byte line per eight lanes and put
+// into MFMA layout with one exchange between lanes i and i ^ 8 (see WaveAttn::issue_k).
+#ifndef FA_K_ROW_LOADS
+#define FA_K_ROW_LOADS 1
+#endif
+
 namespace fa {
 
 struct PagedAttnParams {
@@ -90,6 +96,13 @@ struct WaveAttn {
   static constexpr int NP2 = TPC / 2;             // 32-token P.V steps per chunk
   static constexpr int NR = NDT * 4;              // accumulator values per lane
   static constexpr bool kStream = STREAM;  // non-temporal K/V loads
+  // K rows of one or two 128-byte lines: a load instruction in MFMA layout (lane 16r+i takes
+  // 16 B of row i) would touch half of each of 16 lines, and the memory pipeline pays per line
+  // touched -- measured on a plain streaming probe, 3-5 % of the bandwidth.  Instead a load
+  // takes one whole line of each of eight rows (lane (r, i): row 8h + (i & 7), bytes
+  // 128 L + (i >> 3) * 64 + r * 16 for load c = 2L + h), and k_rows_to_mfma() moves the halves
+  // that sit in the wrong lane across with DPP.  The head-dim <-> k-slot map stays what it was.
+  static constexpr bool kRowLoads = FA_K_ROW_LOADS != 0 && ROWB >= 128;
 
   // Register image of one chunk of K and V.
   struct Chunk {
@@ -268,9 +281,20 @@ struct WaveAttn {
   __device__ __forceinline__ void issue_k(Chunk &R, int kvh, int ci, const Ids &ids) const {
 #pragma unroll
     for (int t = 0; t < TPC; ++t) {
-      const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
+      if constexpr (kRowLoads) {
+        // load c brings line c >> 1 of the rows 8 (c & 1) .. 8 (c & 1) + 7 whole: the lanes (r, i)
+        // and (r, i ^ 8) share a row
+        const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)(i & 7) * p.kv_token_bytes +
+                         (i >> 3) * 64 + r * 16;
 #pragma unroll
-      for (int c = 0; c < KL; ++c) R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + c * 64));
+        for (int c = 0; c < KL; ++c)
+          R.k[t][c] = kv_load<kStream>(
+              reinterpret_cast<const u32x4 *>(kp + (int64_t)(8 * (c & 1)) * p.kv_token_bytes + (c >> 1) * 128));
+      } else {
+        const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
+#pragma unroll
+        for (int c = 0; c < KL; ++c) R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + c * 64));
+      }
     }
   }
   __device__ __forceinline__ void issue_v(Chunk &R, int kvh, int ci, const Ids &ids) const {
@@ -281,6 +305,23 @@ struct WaveAttn {
 #pragma unroll
       for (int e = 0; e < 4; ++e) VLoad<VW, kStream>::ld(R.v[t * 4 + e], vp + e * p.kv_token_bytes);
     }
+  }
+
+  // Row loads -> MFMA layout.  After the loads lane (r, i) holds x = bytes (i>>3)*64 + r*16 .. of
+  // row i & 7 and y = the same bytes of row 8 + (i & 7); it needs bytes r*16 .. and 64 + r*16 .. of
+  // row i.  Lanes i < 8 keep x and take x of lane i + 8; lanes i >= 8 keep y and take y of lane
+  // i - 8: one rotation by eight within each row of 16 lanes, written to half of the lanes.
+  static __device__ __forceinline__ void k_rows_to_mfma(u32x4 &x, u32x4 &y) {
+    constexpr int kRowRor8 = 0x128;  // DPP control: rotate right by 8 within a row of 16 lanes
+    u32x4 a0, a1;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      // bank mask 0xC: lanes 8..15 of each row are written, 0x3: lanes 0..7; the others keep `old`
+      a0[w] = __builtin_amdgcn_update_dpp(x[w], y[w], kRowRor8, 0xF, 0xC, false);
+      a1[w] = __builtin_amdgcn_update_dpp(y[w], x[w], kRowRor8, 0xF, 0x3, false);
+    }
+    x = a0;
+    y = a1;
   }
 
   // K "A" operand of k-step c for one tile: row i = token, 8 head-dim elements.
@@ -318,8 +359,14 @@ struct WaveAttn {
   }
 
   // scores: S^T tile rows are tokens 4r+e of the tile, column i is the head
-  __device__ __forceinline__ Scores qk(const Chunk &R) const {
+  __device__ __forceinline__ Scores qk(Chunk &R) const {
     Scores s;
+    if constexpr (kRowLoads) {
+#pragma unroll
+      for (int t = 0; t < TPC; ++t)
+#pragma unroll
+        for (int c = 0; c < KL; c += 2) k_rows_to_mfma(R.k[t][c], R.k[t][c + 1]);
+    }
 #pragma unroll
     for (int t = 0; t < TPC; ++t) s.v[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
