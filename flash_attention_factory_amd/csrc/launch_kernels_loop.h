@@ -17,8 +17,8 @@ namespace fa {
 // kLoopPersistentMaxSeqs sequences, else grid (kv heads, 1, sequences) with NW wavefronts per
 // work-group.  Kernel time is ADDED to *total_us when the call is timed.
 // KVF selects the cache format: 16-bit, or E5M2 / E4M3 bytes (launch_kernels_fp8_loop.h).
-template <int HEAD_SIZE, typename QT, int KVF>
-inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, const void *key_cache,
+template <int HEAD_SIZE, typename QT, int KVF, bool KROW>
+inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const void *key_cache,
                                               const void *value_cache, const int32_t *block_tables,
                                               const int32_t *context_lens, float scale,
                                               const fa_paged_attention_shape &shape, const Resolved &r,
@@ -47,11 +47,11 @@ inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, cons
       // sequences first, with the next item's first loads issued before each merge.
       constexpr int PW = PersistentLoop<KV8>::waves;
       auto plain = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                     Pipeline<KV8>::tiles_per_chunk, false>;
+                                                     Pipeline<KV8>::tiles_per_chunk, false, 1, KROW>;
       auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                        Pipeline<KV8>::tiles_per_chunk, true>;
+                                                        Pipeline<KV8>::tiles_per_chunk, true, 1, KROW>;
       auto two_tiles = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                         Pipeline<KV8>::tiles_per_chunk, true, 2>;
+                                                         Pipeline<KV8>::tiles_per_chunk, true, 2, KROW>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
       int resident = 0;
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
@@ -61,19 +61,36 @@ inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, cons
       const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
-                            Pipeline<KV8>::tiles_per_chunk, true>,
+                            Pipeline<KV8>::tiles_per_chunk, true, KROW>,
           grid, dim3(NW * 64), 0, p));
     } else {
       const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
-                            Pipeline<KV8>::tiles_per_chunk>,
+                            Pipeline<KV8>::tiles_per_chunk, false, KROW>,
           grid, dim3(NW * 64), 0, p));
     }
     if (r.elapsed_us) FA_HIP_CHECK(timer.accumulate(0, &total_us));
   }
   *total_us_out += total_us;
   return FA_OK;
+}
+
+// Picks how K tiles are loaded (see kRowLoadsLoop16Adjacent): whole lines, except for a 16-bit cache
+// whose token rows are adjacent.
+template <int HEAD_SIZE, typename QT, int KVF>
+inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, const void *key_cache,
+                                              const void *value_cache, const int32_t *block_tables,
+                                              const int32_t *context_lens, float scale,
+                                              const fa_paged_attention_shape &shape, const Resolved &r,
+                                              float *total_us_out) {
+  if constexpr (KVF == kKv16 && !kRowLoadsLoop16Adjacent) {
+    if (shape.kv_token_stride == shape.head_size)
+      return launch_paged_attn_loop_rows<HEAD_SIZE, QT, KVF, false>(out, query, key_cache, value_cache, block_tables,
+                                                                    context_lens, scale, shape, r, total_us_out);
+  }
+  return launch_paged_attn_loop_rows<HEAD_SIZE, QT, KVF, true>(out, query, key_cache, value_cache, block_tables,
+                                                               context_lens, scale, shape, r, total_us_out);
 }
 
 // Whether the persistent kernel takes batches of this shape at all (given few enough sequences).

@@ -96,10 +96,10 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
 // head) pairs; an FP8 cache may bring per-head or per-block scales (p.kv_scale_mode).  Chunks
 // that lie wholly before a sequence's window are skipped; a partition of which a column sees
 // nothing stores an empty partial for it (max -inf, sum 0, zeros).
-template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC, bool MASKS = false>
+template <int D, typename QT, int KVF, bool PART, int NW, int OCC, int TPC, bool MASKS = false, bool KROW = true>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_kernel(const PagedAttnParams p) {
-  using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop, MASKS>;
+  using W = WaveAttn<D, QT, KVF, TPC, PART ? Pipeline<(KVF != 0)>::stream_loads_split : Pipeline<(KVF != 0)>::stream_loads_loop, MASKS, KROW>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   constexpr int CT = W::CT;

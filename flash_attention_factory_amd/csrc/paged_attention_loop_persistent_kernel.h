@@ -40,12 +40,12 @@ constexpr int kLoopPersistentSpinLimit = 1 << 24;
 // on -- and merges and stores for itself.  The groups run the same code on the same chunks at
 // the same time, so K and V come from HBM once and from the cache for the other groups
 // (their loads are not marked non-temporal for that reason).
-template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, int TILES = 1>
+template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, int TILES = 1, bool KROW = true>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   static_assert(TILES == 1 || EXT, "column tiles belong to the extended instances");
   constexpr int NW = NWG / TILES;  // wavefronts that share an item's chunks and merge: one group
-  using W = WaveAttn<D, QT, KVF, TPC, TILES == 1 && Pipeline<(KVF != 0)>::stream_loads_loop, EXT>;
+  using W = WaveAttn<D, QT, KVF, TPC, TILES == 1 && Pipeline<(KVF != 0)>::stream_loads_loop, EXT, KROW>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   using ItemExt = typename W::ItemExt;

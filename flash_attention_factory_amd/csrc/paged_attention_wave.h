@@ -28,6 +28,7 @@
 #define FA_K_ROW_LOADS 1
 #endif
 
+
 namespace fa {
 
 struct PagedAttnParams {
@@ -81,7 +82,8 @@ constexpr int kScaleTensor = 0, kScaleHead = 1, kScaleBlock = 2;  // = fa_kv_sca
 // The MFMA columns then stand for (query token, head) pairs: column i = query token
 // p.query_first + i / G, head i % G of the kv head's group; a launch covers the p.query_count
 // tokens that fit the 16 columns, the host launches once per such group of tokens.
-template <int D, typename QT, int KVF, int TPC, bool STREAM, bool EXT = false>
+// KROW: K tiles are loaded a whole 128-byte line per eight lanes (see kRowLoads below).
+template <int D, typename QT, int KVF, int TPC, bool STREAM, bool EXT = false, bool KROW = true>
 struct WaveAttn {
   static constexpr bool KV8 = KVF != kKv16;
   static constexpr bool kExt = EXT;
@@ -102,7 +104,8 @@ struct WaveAttn {
   // takes one whole line of each of eight rows (lane (r, i): row 8h + (i & 7), bytes
   // 128 L + (i >> 3) * 64 + r * 16 for load c = 2L + h), and k_rows_to_mfma() moves the halves
   // that sit in the wrong lane across with DPP.  The head-dim <-> k-slot map stays what it was.
-  static constexpr bool kRowLoads = FA_K_ROW_LOADS != 0 && ROWB >= 128;
+  static constexpr bool kRowLoads = FA_K_ROW_LOADS != 0 && KROW && ROWB >= 128;
+
 
   // Register image of one chunk of K and V.
   struct Chunk {
@@ -288,8 +291,8 @@ struct WaveAttn {
                          (i >> 3) * 64 + r * 16;
 #pragma unroll
         for (int c = 0; c < KL; ++c)
-          R.k[t][c] = kv_load<kStream>(
-              reinterpret_cast<const u32x4 *>(kp + (int64_t)(8 * (c & 1)) * p.kv_token_bytes + (c >> 1) * 128));
+          R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(
+              kp + (int64_t)(8 * (c & 1)) * p.kv_token_bytes + (c >> 1) * 128));
       } else {
         const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
 #pragma unroll
