@@ -49,6 +49,10 @@ FA_KV_SCALE_TENSOR = 0
 FA_KV_SCALE_HEAD = 1
 FA_KV_SCALE_BLOCK = 2
 
+FA_SCHEDULE_AUTO = 0
+FA_SCHEDULE_GRID = 1
+FA_SCHEDULE_GRID_LDS = 2
+
 FA_MASK_ALIBI = 1
 FA_MASK_SOFTCAP = 2
 FA_MASK_WINDOW = 4
@@ -88,6 +92,7 @@ class Options(ctypes.Structure):
         ("kv_scale_mode", ctypes.c_int32),
         ("k_scales", ctypes.c_void_p),
         ("v_scales", ctypes.c_void_p),
+        ("schedule", ctypes.c_int32),
     ]
 
 

@@ -140,4 +140,4 @@ FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *ke
 
 FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
 
-FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 6; }
+FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 7; }

@@ -17,6 +17,7 @@
 
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
+#include "paged_attention_lds_kernel.h"
 #include "paged_attention_loop_persistent_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
@@ -70,6 +71,7 @@ struct Resolved {
   int32_t kv_scale_mode;  // fa_kv_scale; with a mode other than 0 fp8_scale is 1
   const float *k_scales;
   const float *v_scales;
+  int32_t schedule;  // fa_schedule
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -175,6 +177,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
     r->v_scales = o->v_scales;
     r->fp8_scale = 1.0f;
   }
+  r->schedule = o ? o->schedule : FA_SCHEDULE_AUTO;
+  if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS)
+    return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2)", r->schedule);
   r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   r->elapsed_us = o ? o->elapsed_us : nullptr;
   r->validate_only = o && o->validate_only != 0;

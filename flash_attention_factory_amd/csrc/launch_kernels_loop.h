@@ -33,8 +33,9 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float total_us = 0.f;
-  const bool persistent = kUsePersistentLoop && shape.num_seqs <= kLoopPersistentMaxSeqs &&
-                          shape.num_pool_blocks > 0 && max_ctx < kLoopPersistentMaxContext;
+  const bool persistent = kUsePersistentLoop && r.schedule == FA_SCHEDULE_AUTO &&
+                          shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
+                          max_ctx < kLoopPersistentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
   // columns, or in the persistent form two tiles of 16 held by two halves of every work-group.
   const int per_tile = p.query_count;
@@ -57,6 +58,12 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
       const dim3 grid((unsigned)std::min<int64_t>(resident, items));
       FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
+    } else if (KV8 && HEAD_SIZE == 128 && !ext && r.schedule == FA_SCHEDULE_GRID_LDS) {
+      // grid form, K and V staged through LDS: one work-group of eight wavefronts per compute unit
+      if constexpr (KV8 && HEAD_SIZE == 128) {
+        const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+        FA_HIP_CHECK(timer.launch(paged_attn_lds_kernel<HEAD_SIZE, QT, KVF, false, 8, 2>, grid, dim3(8 * 64), 0, p));
+      }
     } else if (ext) {
       const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
@@ -108,7 +115,7 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
                                         int32_t /*max_context_len: validation only*/,
                                         const fa_paged_attention_shape &shape, const Resolved &r) {
   float total_us = 0.f;
-  if (PersistentLoop<(KVF != kKv16)>::sub_batches && loop_persistent_fits(shape) &&
+  if (PersistentLoop<(KVF != kKv16)>::sub_batches && r.schedule == FA_SCHEDULE_AUTO && loop_persistent_fits(shape) &&
       shape.num_seqs > kLoopPersistentMaxSeqs) {
     const int pieces = (shape.num_seqs + kLoopPersistentMaxSeqs - 1) / kLoopPersistentMaxSeqs;
     const int per = (shape.num_seqs + pieces - 1) / pieces;

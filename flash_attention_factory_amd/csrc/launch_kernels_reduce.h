@@ -38,7 +38,7 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float attention_us = 0.f;
-  const bool segment_form = SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs &&
+  const bool segment_form = SegmentSplit<KV8>::use && r.schedule == FA_SCHEDULE_AUTO && shape.num_seqs <= kSegmentMaxSeqs &&
                             shape.num_pool_blocks > 0 &&
                             (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
@@ -74,6 +74,12 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
         segment_groups = (int)std::min<int64_t>(resident, max_items);
       }
       FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
+    } else if (KV8 && HEAD_SIZE == 128 && !ext && r.schedule == FA_SCHEDULE_GRID_LDS) {
+      // grid form, K and V staged through LDS: one wavefront per partition
+      if constexpr (KV8 && HEAD_SIZE == 128) {
+        const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+        FA_HIP_CHECK(timer.launch(paged_attn_lds_kernel<HEAD_SIZE, QT, KVF, true, 1, 2>, grid, dim3(64), 0, p));
+      }
     } else if (ext) {
       const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
@@ -140,7 +146,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
                                       float *exp_sums, float *max_logits, float *tmp_out,
                                       const fa_paged_attention_shape &shape, const Resolved &r) {
   float us[2] = {0.f, 0.f};
-  if (segment_form_fits<(KVF != kKv16)>(shape) && shape.num_seqs > kSegmentMaxSeqs) {
+  if (r.schedule == FA_SCHEDULE_AUTO && segment_form_fits<(KVF != kKv16)>(shape) && shape.num_seqs > kSegmentMaxSeqs) {
     const int pieces = (shape.num_seqs + kSegmentMaxSeqs - 1) / kSegmentMaxSeqs;
     const int per = (shape.num_seqs + pieces - 1) / pieces;
     const int64_t rows = (int64_t)r.query_len * shape.num_heads;  // (query token, head) rows per sequence

@@ -25,9 +25,10 @@ namespace fa {
 //          max_logits = M (natural-log units), exp_sums = L
 // After the merge wavefront w owns the slice idx in [w*SL, (w+1)*SL) of every lane's NR
 // consecutive head-dim elements and stores it.
+// `lds`: NW * (NR * 64 + 32) floats of LDS the work-group is done with otherwise (unused with NW = 1).
 template <bool PART, int NW, typename W>
 __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p, int lane, int wave,
-                                                int seq, int kvh, int part) {
+                                                int seq, int kvh, int part, float *lds) {
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
   constexpr int D = NDT * 16;
@@ -41,9 +42,9 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
 #pragma unroll
     for (int k = 0; k < SL; ++k) o[k] = wa.acc_at(k);
   } else {
-    __shared__ float sm_m[NW][16];
-    __shared__ float sm_l[NW][16];
-    __shared__ float sm_acc[NW][NR][64];
+    float (*sm_acc)[NR][64] = reinterpret_cast<float (*)[NR][64]>(lds);
+    float (*sm_m)[16] = reinterpret_cast<float (*)[16]>(lds + NW * NR * 64);
+    float (*sm_l)[16] = reinterpret_cast<float (*)[16]>(lds + NW * NR * 64 + NW * 16);
     if (r == 0) {
       sm_m[wave][i] = wa.m;
       sm_l[wave][i] = wa.l;
@@ -175,7 +176,8 @@ paged_attn_kernel(const PagedAttnParams p) {
     wa.pv(R, wa.template soft<true, MASKS>(R, s, ci, tok_end, &ts));
   }
 
-  merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part);
+  __shared__ float merge_lds[NW > 1 ? NW * (W::NR * 64 + 32) : 1];
+  merge_and_store<PART, NW>(wa, p, lane, wave, seq, kvh, part, merge_lds);
 }
 
 }  // namespace fa

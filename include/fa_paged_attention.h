@@ -97,6 +97,17 @@ typedef enum fa_mask { FA_MASK_ALIBI = 1, FA_MASK_SOFTCAP = 2, FA_MASK_WINDOW = 
  *   FA_KV_SCALE_BLOCK  k_scales, v_scales [num_pool_blocks, num_kv_heads] fp32, one scale per
  *                      physical block and kv head (num_pool_blocks must be given)
  * K^ = dequant(K) * k_scale, V^ = dequant(V) * v_scale.  Scales must be finite and positive. */
+/* How the work is laid over the GPU.  FA_SCHEDULE_AUTO picks the fastest form for the batch: for
+ * batches of up to a few hundred sequences resident work-groups that walk the (sequence, kv head)
+ * items -- and, in the split path, write one partial per SEGMENT of several partitions.
+ * FA_SCHEDULE_GRID is upstream's own decomposition, one work-group per (sequence, kv head) and,
+ * in the split path, per partition (paged_attention_kernel_loop.hpp:602-607,
+ * paged_attention_kernel_v2.hpp:562-569): every live slot of exp_sums / max_logits / tmp_out then
+ * holds exactly what upstream stores there.  FA_SCHEDULE_GRID_LDS is the grid form with K and V
+ * staged through LDS by direct-to-LDS loads (FP8 entries, head size 128, no score modifiers;
+ * anything else falls back to FA_SCHEDULE_GRID).  `out` is the same under all three. */
+typedef enum fa_schedule { FA_SCHEDULE_AUTO = 0, FA_SCHEDULE_GRID = 1, FA_SCHEDULE_GRID_LDS = 2 } fa_schedule;
+
 typedef enum fa_kv_scale { FA_KV_SCALE_TENSOR = 0, FA_KV_SCALE_HEAD = 1, FA_KV_SCALE_BLOCK = 2 } fa_kv_scale;
 
 /* Shapes and strides that upstream reads off the torch tensors
@@ -155,6 +166,7 @@ typedef struct fa_paged_attention_options {
                                  arrays below are read */
   const float *k_scales;      /* device, fp32, shaped as kv_scale_mode says; NULL with mode 0 */
   const float *v_scales;
+  int32_t schedule;           /* fa_schedule; 0 = the library chooses */
 } fa_paged_attention_options;
 
 /* Single-pass kernel: no scratch.  One launch for a decode batch of up to 128 sequences; larger

@@ -29,14 +29,15 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 6
+    assert L.fa_paged_attention_abi_version() == 7
 
 
 def test_struct_layouts_match_header():
     # field order and sizes of the two structs as the header lays them out
     assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
     assert _cabi.Shape.kv_block_stride.offset == 32
-    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4 + 8 + 8
+    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4 + 8 + 8 + 8
+    assert _cabi.Options.schedule.offset == 80
     assert _cabi.Options.kv_scale_mode.offset == 60
     assert _cabi.Options.k_scales.offset == 64 and _cabi.Options.v_scales.offset == 72
     assert _cabi.Options.query_len.offset == 56
@@ -60,8 +61,9 @@ def _shape(**kw):
 
 def _call(L, split=False, fp8=False, shape=None, ptr=0x1000, scratch=0x1000, max_ctx=0, fp8_format=0,
           mask_flags=0, alibi=None, softcap=0.0, window_left=0, query_len=0, scale_mode=0, k_scales=None,
-          v_scales=None):
+          v_scales=None, schedule=0):
     op = _cabi.Options()
+    op.schedule = schedule
     op.kv_scale_mode, op.k_scales, op.v_scales = scale_mode, k_scales, v_scales
     op.query_len = query_len
     op.validate_only = 1
@@ -216,6 +218,15 @@ def test_kv_scale_argument_checks(L):
     assert _kv_write(L, scale_mode=BLOCK, k_scales=0x1000)[0] == _cabi.FA_ERR_NULL_POINTER
     assert _kv_write(L, scale_mode=9, k_scales=0x1000, v_scales=0x1000)[0] == _cabi.FA_ERR_BAD_SHAPE
     assert _kv_write(L, scale_mode=9, cache_dtype=_cabi.FA_KV_CACHE_16BIT)[0] == _cabi.FA_OK
+
+
+def test_schedule_values(L):
+    for split in (False, True):
+        for fp8 in (False, True):
+            for schedule in (0, 1, 2):  # the LDS form falls back to the grid form where it does not apply
+                assert _call(L, split=split, fp8=fp8, schedule=schedule)[0] == _cabi.FA_OK
+            code, text = _call(L, split=split, fp8=fp8, schedule=3)
+            assert code == _cabi.FA_ERR_BAD_SHAPE and "schedule" in text
 
 
 def test_static_scratch_rejects_what_does_not_fit(L):

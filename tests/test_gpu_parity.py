@@ -23,11 +23,11 @@ def _dev():
     return torch.device("cuda:0")
 
 
-def _run(w_cpu, kernel, max_context_len=None, **kw):
+def _run(w_cpu, kernel, max_context_len=None, schedule=0, **kw):
     from flash_attention_factory_amd import runner
     w = w_cpu.to(_dev())
     bufs = runner.alloc_buffers(w, **kw)
-    times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len)
+    times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len, schedule=schedule)
     torch.cuda.synchronize()
     return bufs, times
 
@@ -116,6 +116,40 @@ def test_partition_scratch_matches_kernel_model(oracle, fp8):
         torch.testing.assert_close(g_es[s, :, :live], es[s, :, :live], atol=1e-4, rtol=1e-4)
         torch.testing.assert_close(g_tmp[s, :, :live], tmp[s, :, :live], atol=2e-3, rtol=1e-2)
         assert torch.isnan(g_ml[s, :, live:]).all() and torch.isnan(g_tmp[s, :, live:]).all()
+
+
+@pytest.mark.parametrize("schedule", [1, 2])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_schedule_option(oracle, fp8, schedule):
+    """options->schedule: the grid form (upstream's own decomposition, one work-group per (sequence, kv
+    head[, partition])) and, for FP8 caches, its variant with K/V staged through LDS by direct-to-LDS
+    loads -- on a batch the library would by itself run in the persistent forms.  Same `out`; in the
+    split path every live slot of the scratch arrays holds upstream's per-partition values."""
+    w = W.make_config(4 if fp8 else 2, num_seqs=5, pool_blocks=4096, lens=[1, 33, 2048, 1537, 700])
+    if not fp8:
+        w = W.make_config(2, num_seqs=5, pool_blocks=4096, lens=[1, 33, 2048, 1537, 700], layout=W.TOKEN_MAJOR)
+    w.sinks = torch.linspace(-1, 2, w.num_heads).to(w.query.dtype)
+    for kernel in ("loop", "reduce"):
+        kernel = ("fp8_" if fp8 else "") + kernel
+        bufs, _ = _run(w, kernel, schedule=schedule)
+        _check(bufs.out, w, oracle, f"{w.name}/{kernel}/schedule{schedule}")
+        if "reduce" in kernel:
+            es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=w.partition_size,
+                                      max_num_partitions=w.max_num_partitions)
+            for s in range(w.num_seqs):
+                live = math.ceil(int(w.context_lens[s]) / w.partition_size)
+                torch.testing.assert_close(bufs.max_logits[s, :, :live].cpu(), ml[s, :, :live], atol=1e-4, rtol=1e-5)
+                torch.testing.assert_close(bufs.exp_sums[s, :, :live].cpu(), es[s, :, :live], atol=1e-4, rtol=1e-4)
+                torch.testing.assert_close(bufs.tmp_out[s, :, :live].cpu(), tmp[s, :, :live], atol=2e-3, rtol=1e-2)
+                assert torch.isnan(bufs.max_logits[s, :, live:]).all()
+
+
+def test_lds_staged_kernel_full_size(oracle):
+    """The LDS-staged grid kernel on the whole FP8 loop configuration, both layouts, and E4M3 bytes."""
+    for kw in (dict(), dict(layout=W.TOKEN_MAJOR), dict(fp8_dtype=torch.float8_e4m3fn)):
+        w = W.make_config(3, **kw)
+        bufs, _ = _run(w, "fp8_loop", schedule=2)
+        _check(bufs.out, w, oracle, f"{w.name}/lds/{kw}")
 
 
 def test_edge_cases(oracle):
