@@ -136,6 +136,16 @@ def set_kv_scales(op: "Options", k_scales, v_scales, num_kv_heads: int, num_pool
     op.v_scales = v_scales.data_ptr()
 
 
+def require_same_device(anchor_name: str, anchor, named_tensors) -> None:
+    """Every tensor whose pointer goes to a kernel must live on the anchor tensor's device: a host
+    pointer in a kernel argument is a GPU memory fault, not an exception.  None entries are skipped."""
+    for name, t in named_tensors:
+        if t is not None and t.device != anchor.device:
+            raise PagedAttentionError(FA_ERR_BAD_SHAPE,
+                                      f"{name} is on {t.device}, {anchor_name} on {anchor.device}: every tensor "
+                                      f"must live on the device of {anchor_name}")
+
+
 class PagedAttentionError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"[fa_status {code}] {message}")

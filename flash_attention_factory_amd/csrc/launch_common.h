@@ -12,8 +12,10 @@
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "../../include/fa_paged_attention.h"
 #include "paged_attention_kernel.h"
@@ -45,6 +47,39 @@ inline fa_status fail(fa_status code, const char *fmt, ...) {
       return ::fa::fail(FA_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(e_));     \
   } while (0)
 
+// The status word of the persistent kernels: a wavefront that exhausts its spin limit while it
+// waits for the other wavefronts of its work-group stores kStatusSpinLimit here and goes on (so
+// the grid drains) with a result that is wrong.  One word per GPU, in device memory; as with any
+// __device__ variable the name is only a handle on the host, the address on the current device
+// comes from hipGetSymbolAddress, once per device.
+static __device__ int32_t kernel_status_word;
+
+inline fa_status kernel_status_of_current_device(int32_t **word) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mutex;
+  static int32_t *address[kMaxDevices];  // nullptr until the device's first launch
+  int dev = 0;
+  FA_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(FA_ERR_RUNTIME, "device %d is beyond the %d devices this library serves", dev, kMaxDevices);
+  std::lock_guard<std::mutex> guard(mutex);
+  if (address[dev] == nullptr) {
+    void *a = nullptr;
+    FA_HIP_CHECK(hipGetSymbolAddress(&a, HIP_SYMBOL(kernel_status_word)));
+    address[dev] = static_cast<int32_t *>(a);
+  }
+  *word = address[dev];
+  return FA_OK;
+}
+
+// FA_DEBUG_SPIN_LIMIT in the environment replaces the spin limit of the persistent kernels: the way
+// to see the give-up path run (a limit of 0 makes every merge go ahead without waiting) while every
+// kernel still ends normally.
+inline int32_t spin_limit_of_this_call() {
+  const char *text = getenv("FA_DEBUG_SPIN_LIMIT");
+  return text ? (int32_t)atoi(text) : kLoopPersistentSpinLimit;
+}
+
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 inline int ilog2(int32_t v) {
   int s = 0;
@@ -72,6 +107,8 @@ struct Resolved {
   const float *k_scales;
   const float *v_scales;
   int32_t schedule;  // fa_schedule
+  int32_t *status;   // status word of the current device (nullptr with validate_only)
+  int32_t spin_limit;
   hipStream_t stream;
   float *elapsed_us;
   bool validate_only;
@@ -103,8 +140,6 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   if (s->num_seqs <= 0 || s->num_heads <= 0 || s->num_kv_heads <= 0 || s->max_blocks_per_seq <= 0)
     return fail(FA_ERR_BAD_SHAPE, "num_seqs, num_heads, num_kv_heads and max_blocks_per_seq must be positive");
   if (s->num_pool_blocks < 0) return fail(FA_ERR_BAD_SHAPE, "num_pool_blocks must be >= 0");
-  if (s->num_seqs > 65535)
-    return fail(FA_ERR_BAD_SHAPE, "num_seqs %d exceeds the grid limit 65535", s->num_seqs);
   if (s->num_heads % s->num_kv_heads != 0)
     return fail(FA_ERR_UNSUPPORTED_GROUP, "Unsupported number of queries per token: num_heads %d is "
                                           "not a multiple of num_kv_heads %d", s->num_heads, s->num_kv_heads);
@@ -184,7 +219,27 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->elapsed_us = o ? o->elapsed_us : nullptr;
   r->validate_only = o && o->validate_only != 0;
   r->sinks = o ? o->sinks : nullptr;
+  r->status = nullptr;
+  r->spin_limit = spin_limit_of_this_call();
+  if (!r->validate_only) return kernel_status_of_current_device(&r->status);
   return FA_OK;
+}
+
+// After a timed call (which has synchronised anyway): did a kernel of this GPU give up a wait?
+// Reads the status word, clears it, and turns a set word into FA_ERR_RUNTIME.  Asynchronous calls
+// do not look: the word stays set until the next timed call on the device reports it.
+inline fa_status report_kernel_status(const Resolved &r) {
+  if (!r.elapsed_us || !r.status) return FA_OK;
+  int32_t seen = 0;
+  FA_HIP_CHECK(hipMemcpyAsync(&seen, r.status, sizeof(seen), hipMemcpyDeviceToHost, r.stream));
+  FA_HIP_CHECK(hipStreamSynchronize(r.stream));
+  if (seen == 0) return FA_OK;
+  const int32_t zero = 0;
+  FA_HIP_CHECK(hipMemcpyAsync(r.status, &zero, sizeof(zero), hipMemcpyHostToDevice, r.stream));
+  FA_HIP_CHECK(hipStreamSynchronize(r.stream));
+  return fail(FA_ERR_RUNTIME, "a wavefront gave up waiting for the other wavefronts of its work-group (spin limit %d, "
+                              "status %d): the output of this or an earlier call on this GPU is not valid",
+              r.spin_limit, seen);
 }
 
 inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits, const void *query,
@@ -223,6 +278,8 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.partition_size = r.partition_size;
   p.block_shift = ilog2(s.block_size);
   p.max_block_id = s.num_pool_blocks > 0 ? s.num_pool_blocks - 1 : INT32_MAX;
+  p.spin_limit = r.spin_limit;
+  p.status = r.status;
   p.kv_block_bytes = s.kv_block_stride * r.kv_elem_bytes;
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;

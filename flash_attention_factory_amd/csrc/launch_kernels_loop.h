@@ -115,9 +115,14 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
                                         int32_t /*max_context_len: validation only*/,
                                         const fa_paged_attention_shape &shape, const Resolved &r) {
   float total_us = 0.f;
-  if (PersistentLoop<(KVF != kKv16)>::sub_batches && r.schedule == FA_SCHEDULE_AUTO && loop_persistent_fits(shape) &&
-      shape.num_seqs > kLoopPersistentMaxSeqs) {
-    const int pieces = (shape.num_seqs + kLoopPersistentMaxSeqs - 1) / kLoopPersistentMaxSeqs;
+  // most sequences one launch takes: what the persistent kernel ranks, or what the grid's third
+  // dimension holds
+  constexpr int kGridMaxSeqs = 65535;
+  const bool persistent_pieces = PersistentLoop<(KVF != kKv16)>::sub_batches && r.schedule == FA_SCHEDULE_AUTO &&
+                                 loop_persistent_fits(shape) && shape.num_seqs > kLoopPersistentMaxSeqs;
+  const int most = persistent_pieces ? kLoopPersistentMaxSeqs : kGridMaxSeqs;
+  if (shape.num_seqs > most) {
+    const int pieces = (shape.num_seqs + most - 1) / most;
     const int per = (shape.num_seqs + pieces - 1) / pieces;
     const int64_t row_bytes = (int64_t)r.query_len * shape.num_heads * shape.head_size * 2;  // of query and out
     for (int s0 = 0; s0 < shape.num_seqs; s0 += per) {
@@ -135,7 +140,7 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
     if (st != FA_OK) return st;
   }
   if (r.elapsed_us) r.elapsed_us[0] = total_us;
-  return FA_OK;
+  return report_kernel_status(r);
 }
 
 template <bool KV8>

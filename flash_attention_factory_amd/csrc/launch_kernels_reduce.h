@@ -146,8 +146,14 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
                                       float *exp_sums, float *max_logits, float *tmp_out,
                                       const fa_paged_attention_shape &shape, const Resolved &r) {
   float us[2] = {0.f, 0.f};
-  if (r.schedule == FA_SCHEDULE_AUTO && segment_form_fits<(KVF != kKv16)>(shape) && shape.num_seqs > kSegmentMaxSeqs) {
-    const int pieces = (shape.num_seqs + kSegmentMaxSeqs - 1) / kSegmentMaxSeqs;
+  // most sequences one launch takes: what the segment kernel lists, or what the grid's third
+  // dimension holds
+  constexpr int kGridMaxSeqs = 65535;
+  const bool segment_pieces = r.schedule == FA_SCHEDULE_AUTO && segment_form_fits<(KVF != kKv16)>(shape) &&
+                              shape.num_seqs > kSegmentMaxSeqs;
+  const int most = segment_pieces ? kSegmentMaxSeqs : kGridMaxSeqs;
+  if (shape.num_seqs > most) {
+    const int pieces = (shape.num_seqs + most - 1) / most;
     const int per = (shape.num_seqs + pieces - 1) / pieces;
     const int64_t rows = (int64_t)r.query_len * shape.num_heads;  // (query token, head) rows per sequence
     const int64_t row_bytes = rows * shape.head_size * 2;           // of query and out
@@ -171,7 +177,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
     r.elapsed_us[0] = us[0];
     r.elapsed_us[1] = us[1];
   }
-  return FA_OK;
+  return report_kernel_status(r);
 }
 
 template <bool KV8>

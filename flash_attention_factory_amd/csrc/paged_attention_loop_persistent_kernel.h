@@ -30,8 +30,11 @@ constexpr int kLoopPersistentMaxSeqs = 128;
 constexpr int kLoopPersistentMaxContext = 1 << 24;  // lengths are packed into 24 bits of a sort key
 // Upper bound on the polls of one wait for the other wavefronts of a work-group (each poll
 // sleeps ~64 cycles).  Never reached in a correct run -- every wavefront publishes every
-// item -- it only turns a would-be hang into a wrong answer that the tests catch.
+// item -- it only turns a would-be hang into a wrong answer plus a flag in the launch's status
+// word, which a timed call reports as FA_ERR_RUNTIME.
 constexpr int kLoopPersistentSpinLimit = 1 << 24;
+// What a kernel leaves in the status word (PagedAttnParams::status) when it gave up such a wait.
+constexpr int32_t kStatusSpinLimit = 1;
 
 //
 // TILES (extended instances): column tiles per launch.  The NWG wavefronts of a work-group then
@@ -166,11 +169,18 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   auto finish = [&](int item, int seq, int kvh, float out_mul) {
     const int b = item & 1;
     const int target = NW * ((item >> 1) + 1);
-    for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
+    bool arrived = false;
+    for (int spin = 0; spin < p.spin_limit; ++spin) {
       const int seen = __hip_atomic_load(&sm_arrived[tile][b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+      if (__builtin_amdgcn_readfirstlane(seen) >= target) {
+        arrived = true;
+        break;
+      }
       __builtin_amdgcn_s_sleep(1);
     }
+    // Gave up: what follows merges states that are not all there, so the result is wrong; say so in
+    // the status word (one lane, a plain vector store) and carry on, so that the grid still drains.
+    if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     float M = -INFINITY;
 #pragma unroll

@@ -192,11 +192,18 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   auto finish = [&](int n, const Item &it, float out_mul) {
     const int b = n & 1;
     const int target = NW * ((n >> 1) + 1);
-    for (int spin = 0; spin < kLoopPersistentSpinLimit; ++spin) {
+    bool arrived = false;
+    for (int spin = 0; spin < p.spin_limit; ++spin) {
       const int seen = __hip_atomic_load(&sm_arrived[tile][b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+      if (__builtin_amdgcn_readfirstlane(seen) >= target) {
+        arrived = true;
+        break;
+      }
       __builtin_amdgcn_s_sleep(1);
     }
+    // Gave up: what follows merges states that are not all there, so the result is wrong; say so in
+    // the status word (one lane, a plain vector store) and carry on, so that the grid still drains.
+    if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     float M = -INFINITY;
 #pragma unroll

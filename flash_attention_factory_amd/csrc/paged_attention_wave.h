@@ -69,6 +69,10 @@ struct PagedAttnParams {
   int32_t kv_scale_mode;        // kScaleTensor / kScaleHead / kScaleBlock
   const float *k_scales;        // [Hk] or [pool blocks, Hk] fp32
   const float *v_scales;
+  // persistent kernels: polls a wavefront spends on one wait for the other wavefronts of its
+  // work-group before it gives up, and the device word in which it says so (see launch_common.h)
+  int32_t spin_limit;
+  int32_t *status;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
@@ -454,8 +458,10 @@ struct WaveAttn {
     // k-slots (r, e) of step pr = this lane's eight tokens of the step, rounded to the q
     // dtype (paged_attention_kernel_loop.hpp:404-407)
     if constexpr (MASKS && KV8) {  // per-block V scales ride on the probabilities (1.0 otherwise)
+      // by select: a tile past the context takes its block id from a clamped or unused table
+      // column, and the scale of a block nobody wrote may be anything, NaN included
 #pragma unroll
-      for (int e = 0; e < NT; ++e) t[e] *= ts->v[e >> 2];
+      for (int e = 0; e < NT; ++e) t[e] = t[e] == 0.f ? 0.f : t[e] * ts->v[e >> 2];
     }
     Probs pb;
 #pragma unroll

@@ -11,6 +11,7 @@ the contiguous ``[blocks, block_size, kv_heads, head_size]`` tensor.
 from __future__ import annotations
 
 import ctypes
+import warnings
 from typing import List, Optional
 
 import torch
@@ -18,6 +19,7 @@ import torch
 from .. import _cabi
 
 _scratch = {}
+_warned_scratch = False
 
 
 def _fp32_scratch(tem_output: torch.Tensor, shape) -> torch.Tensor:
@@ -28,10 +30,18 @@ def _fp32_scratch(tem_output: torch.Tensor, shape) -> torch.Tensor:
         want *= n
     if tem_output.dtype == torch.float32 and tem_output.numel() == want and tem_output.is_contiguous():
         return tem_output
-    key = (tem_output.device, tuple(shape))
+    global _warned_scratch
+    if not _warned_scratch:
+        _warned_scratch = True
+        warnings.warn("tem_output is not a contiguous fp32 tensor of the scratch shape (upstream keeps it in the "
+                      "query dtype): the kernels use a cached fp32 workspace of their own instead, allocated on "
+                      "first use and shared by every call on this stream -- pass fp32 scratch to avoid it",
+                      RuntimeWarning, stacklevel=4)
+    key = (tem_output.device, torch.cuda.current_stream(tem_output.device).cuda_stream, tuple(shape))
     buf = _scratch.get(key)
     if buf is None:
-        _scratch.clear()
+        if len(_scratch) >= 8:
+            _scratch.clear()
         buf = torch.empty(shape, dtype=torch.float32, device=tem_output.device)
         _scratch[key] = buf
     return buf
@@ -51,6 +61,13 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     L = _cabi.load()
     if not query.is_cuda:
         raise RuntimeError("paged attention runs on the GPU only: `query` is not a device tensor")
+    # every pointer handed to the kernels must be a device pointer on the query's device: a host
+    # tensor here would be a GPU memory fault, not an exception
+    tensors = [("output", output), ("key_cache", key_cache), ("value_cache", value_cache),
+               ("block_tables", block_tables), ("context_lens", context_lens), ("sinks", sinks)]
+    if split and not static_scratch_partitions:
+        tensors += [("max_logits", max_logits), ("exp_sums", exp_sums), ("tem_output", tem_output)]
+    _cabi.require_same_device("query", query, tensors)
     for name, t in (("query", query), ("output", output), ("block_tables", block_tables),
                     ("context_lens", context_lens)):
         if not t.is_contiguous():
@@ -76,6 +93,15 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
         (S, H, D), QL = query.shape, 1
     if output.shape != query.shape:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE, "output must have the shape of query")
+    if block_tables.dim() != 2 or block_tables.size(0) != S or context_lens.numel() != S:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
+                                        f"block_tables must be [{S}, max_blocks_per_seq] and context_lens [{S}]")
+    if key_cache.size(3) != D:
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_HEAD_OR_BLOCK_SIZE,
+                                        f"caches hold rows of {key_cache.size(3)} elements, query heads of {D}")
+    if sinks is not None and (sinks.dtype != query.dtype or sinks.numel() != H or not sinks.is_contiguous()):
+        raise _cabi.PagedAttentionError(_cabi.FA_ERR_BAD_SHAPE,
+                                        f"sinks must be a contiguous [{H}] tensor of the query dtype")
     sh = _cabi.Shape()
     sh.num_seqs, sh.num_heads, sh.head_size = S, H, D
     sh.num_kv_heads = key_cache.size(2)

@@ -29,6 +29,8 @@ def run(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_c
     L = _cabi.load()
     if not key.is_cuda:
         raise RuntimeError("the KV-cache writer runs on the GPU only: `key` is not a device tensor")
+    _cabi.require_same_device("key", key, (("value", value), ("key_cache", key_cache), ("value_cache", value_cache),
+                                           ("slot_mapping", slot_mapping)))
     if key.dtype not in (torch.float16, torch.bfloat16) or value.dtype != key.dtype:
         raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE, "key/value must both be fp16 or both bf16")
     if key.dim() != 3 or key.stride(2) != 1 or value.shape != key.shape or value.stride() != key.stride():

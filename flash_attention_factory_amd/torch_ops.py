@@ -25,6 +25,12 @@ FP8 operators and ``kv_cache_write`` take ``k_scales`` / ``v_scales`` (fp32 ``[k
 ``[blocks, kv_heads]``) in place of the scalar ``fp8_scale``.  ``query`` / ``out`` may be
 ``[seqs, query_len, heads, head_size]``: several causal query tokens per sequence.
 
+SCRATCH CAPACITY of the reduce operators: ``exp_sums.size(-1)`` partitions of ``partition_size`` tokens must
+cover the longest context of the batch.  The kernels cannot raise an error: a longer context is attended
+over its first ``partitions * partition_size`` tokens only.  Pass ``max_context_len`` (the longest
+context, known on the host) and the call fails with FA_ERR_PARTITION_OVERFLOW instead; with the default
+0 nothing is checked.
+
 Caches are ``[blocks, block_size, kv_heads, head_size]`` views as in ``lib.*.run``; every
 output is an argument the operator mutates, nothing is allocated.  Importing this module
 registers the operators; there is no CPU implementation.
@@ -79,12 +85,12 @@ def paged_attention_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tm
                            key_cache: Tensor, value_cache: Tensor, block_tables: Tensor, context_lens: Tensor,
                            scale: float, partition_size: int = 0, sinks: Optional[Tensor] = None,
                            alibi_slopes: Optional[Tensor] = None, softcap: float = 0.0,
-                           window_left: int = -1) -> None:
+                           window_left: int = -1, max_context_len: int = 0) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
     _reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
-                context_lens, _group(query, key_cache), scale, key_cache.size(1), 0, alibi_slopes, sinks, softcap,
-                partition_size=partition_size, timed=False, **_modifiers(alibi_slopes, softcap, window_left))
+                context_lens, _group(query, key_cache), scale, key_cache.size(1), max_context_len, alibi_slopes, sinks,
+                softcap, partition_size=partition_size, timed=False, **_modifiers(alibi_slopes, softcap, window_left))
 
 
 @torch.library.custom_op(f"{_NS}::paged_attention_fp8_reduce",
@@ -94,12 +100,12 @@ def paged_attention_fp8_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor
                                context_lens: Tensor, scale: float, fp8_scale: float, partition_size: int = 0,
                                sinks: Optional[Tensor] = None, alibi_slopes: Optional[Tensor] = None,
                                softcap: float = 0.0, window_left: int = -1, k_scales: Optional[Tensor] = None,
-                               v_scales: Optional[Tensor] = None) -> None:
+                               v_scales: Optional[Tensor] = None, max_context_len: int = 0) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
     _fp8_reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
-                    context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), 0, alibi_slopes,
-                    sinks, softcap, partition_size=partition_size, timed=False, k_scales=k_scales,
+                    context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), max_context_len,
+                    alibi_slopes, sinks, softcap, partition_size=partition_size, timed=False, k_scales=k_scales,
                     v_scales=v_scales, **_modifiers(alibi_slopes, softcap, window_left))
 
 

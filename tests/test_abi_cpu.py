@@ -147,6 +147,19 @@ def test_run_shim_rejects_cpu_tensors():
         runner.run_workload(w, "loop")
 
 
+def test_every_tensor_must_be_on_the_anchor_device():
+    # the check the run shims make before any pointer reaches a kernel, on devices a CPU box has
+    import torch
+    q = torch.empty(2, device="meta")
+    ok = torch.empty(2, device="meta")
+    host = torch.empty(2)
+    _cabi.require_same_device("query", q, [("output", ok), ("sinks", None)])
+    for name in ("output", "key_cache", "value_cache", "block_tables", "context_lens", "sinks", "max_logits",
+                 "exp_sums", "tem_output", "slot_mapping"):
+        with pytest.raises(_cabi.PagedAttentionError, match=name):
+            _cabi.require_same_device("query", q, [("other", ok), (name, host)])
+
+
 def test_workload_generators_are_deterministic():
     import torch
     from flash_attention_factory_amd import workloads as W

@@ -243,3 +243,40 @@ def test_block_scales_in_every_scheduling_form(oracle):
             unit = ref[live].abs().max()
             torch.testing.assert_close(got[live] / unit, ref[live] / unit, atol=ATOL, rtol=RTOL,
                                        msg=lambda m: f"S={S} {kernel}: {m}")
+
+
+def test_scales_of_unused_blocks_may_be_anything(oracle):
+    """A tile wholly past a context takes its block id from a clamped or padding column of the table;
+    that block's scales (and bytes) belong to nobody and may be NaN.  The V scale is applied by
+    select, like the K/V tail itself: loop, segment and grid forms, block sizes 16 and 32."""
+    for S, seed, block_size, schedule in ((40, 81, 16, 0), (40, 82, 32, 0), (9, 83, 16, 1), (300, 84, 16, 0)):
+        gen = torch.Generator().manual_seed(seed)
+        lens = torch.randint(1, 900, (S,), generator=gen)
+        lens[0], lens[1], lens[2] = 1, 17, 16 * 7 + 3  # contexts that end inside the first tile of a chunk
+        w = W.make_test_shaped(batch_size=S, nheads=8, nheads_k=2, d=128, seqlen_k=900, varlen=False, has_sinks=False,
+                               fp8=True, block_size=block_size, seed=seed)
+        w.context_lens = lens.to(torch.int32)
+        NB = w.key_cache.shape[0]
+        used = torch.zeros(NB, dtype=torch.bool)
+        cols = torch.arange(w.block_tables.shape[1])
+        spare = None
+        for s in range(S):
+            n = -(-int(lens[s]) // block_size)
+            used[w.block_tables[s, :n].long()] = True
+        spare = int((~used).nonzero()[0])
+        for s in range(S):  # every column past the context points at a block nobody uses
+            n = -(-int(lens[s]) // block_size)
+            w.block_tables[s, n:] = spare
+        ks, vs = _scales((NB, 2), seed, 0.2, 3.0), _scales((NB, 2), seed + 1, 0.01, 3.0)
+        ks[~used], vs[~used] = float("nan"), float("nan")
+        kb, vb = w.key_cache.view(torch.uint8), w.value_cache.view(torch.uint8)
+        kb[~used], vb[~used] = 0x7f, 0x7f  # NaN bytes
+        ref = _ref(oracle, w, k_scales=ks, v_scales=vs)
+        assert torch.isfinite(ref).all()
+        wd = w.to(_dev())
+        for kernel in ("fp8_loop", "fp8_reduce"):
+            got = _call(wd, kernel, k_scales=ks.to(_dev()), v_scales=vs.to(_dev()), schedule=schedule).float().cpu()
+            assert torch.isfinite(got).all(), (S, block_size, kernel)
+            unit = ref.abs().max()
+            torch.testing.assert_close(got / unit, ref / unit, atol=ATOL, rtol=RTOL,
+                                       msg=lambda m: f"S={S} B={block_size} {kernel}: {m}")

@@ -453,3 +453,83 @@ def test_whole_upstream_grid(oracle, heads, fp8):
                 _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
             n += 1
     assert n == len(UPSTREAM_SHORT) * 16 + len(UPSTREAM_LONG) * (16 if everything else 1)
+
+
+def test_run_rejects_host_tensors_and_mismatched_shapes():
+    """Nothing reaches a kernel unless it lives on the query's device and has the shape the kernel
+    assumes: a host block table or length array would be a GPU memory fault, not an exception."""
+    from flash_attention_factory_amd import _cabi, runner
+    from flash_attention_factory_amd.lib import kv_cache_write, paged_attention_reduce
+    w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=300, varlen=True, has_sinks=True).to(_dev())
+    bufs = runner.alloc_buffers(w)
+    good = dict(max_logits=bufs.max_logits, exp_sums=bufs.exp_sums, tem_output=bufs.tmp_out, output=bufs.out,
+                key_cache=w.key_cache, value_cache=w.value_cache, block_tables=w.block_tables,
+                context_lens=w.context_lens, sinks=w.sinks)
+
+    def call(**over):
+        a = dict(good, **over)
+        return paged_attention_reduce.run(a["max_logits"], a["exp_sums"], a["tem_output"], a["output"], None, w.query,
+                                          a["key_cache"], a["value_cache"], a["block_tables"], a["context_lens"], 4,
+                                          w.scale, w.block_size, 300, None, a["sinks"], 0.0)
+    call()
+    for name in good:
+        with pytest.raises(_cabi.PagedAttentionError, match=name):
+            call(**{name: good[name].cpu()})
+    with pytest.raises(_cabi.PagedAttentionError, match="block_tables"):
+        call(block_tables=w.block_tables[:1].contiguous())
+    with pytest.raises(_cabi.PagedAttentionError, match="context_lens"):
+        call(context_lens=w.context_lens[:1].contiguous())
+    with pytest.raises(_cabi.PagedAttentionError, match="sinks"):
+        call(sinks=w.sinks.float())
+    with pytest.raises(_cabi.PagedAttentionError, match="sinks"):
+        call(sinks=w.sinks[:4].contiguous())
+    with pytest.raises(_cabi.PagedAttentionError, match="rows of 64"):
+        call(key_cache=w.key_cache[..., :64], value_cache=w.value_cache[..., :64])
+    key = torch.zeros((3, 2, 128), dtype=torch.float16, device=_dev())
+    slots = torch.tensor([0, 1, 2], device=_dev())
+    kv_cache_write.run(key, key, w.key_cache, w.value_cache, slots)
+    for over in (dict(value=key.cpu()), dict(key_cache=w.key_cache.cpu()), dict(value_cache=w.value_cache.cpu()),
+                 dict(slot_mapping=slots.cpu())):
+        a = dict(dict(value=key, key_cache=w.key_cache, value_cache=w.value_cache, slot_mapping=slots), **over)
+        with pytest.raises(_cabi.PagedAttentionError, match=next(iter(over))):
+            kv_cache_write.run(key, a["value"], a["key_cache"], a["value_cache"], a["slot_mapping"])
+
+
+def test_seventy_thousand_sequences(oracle):
+    """More sequences than a grid dimension holds (65535): every path cuts the batch into launches."""
+    S = 70000
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.randint(0, 40, (S,), generator=gen)
+    for fp8 in (False, True):
+        w = W.make_test_shaped(batch_size=S, nheads=2, nheads_k=1, d=64, seqlen_k=48, varlen=False, has_sinks=False,
+                               fp8=fp8, block_size=16, seed=9)
+        w.context_lens = lens.to(torch.int32)
+        w.partition_size = 256
+        _, ref32 = call_oracle(oracle.attention_ref, w, want_f32=True)
+        live = lens > 0
+        for kernel, schedule in (("loop", 0), ("loop", 1), ("reduce", 0), ("reduce", 1)):
+            bufs, _ = _run(w, ("fp8_" if fp8 else "") + kernel, schedule=schedule)
+            got = bufs.out.float().cpu()
+            assert (got[~live] == 0).all()
+            torch.testing.assert_close(got[live], ref32[live], atol=ATOL, rtol=RTOL,
+                                       msg=lambda m: f"fp8={fp8} {kernel} schedule {schedule}: {m}")
+
+
+def test_exhausted_spin_limit_is_reported(oracle):
+    """A wavefront of a persistent kernel that gives up waiting for its work-group sets a status word
+    and lets the grid drain; the timed call returns FA_ERR_RUNTIME.  FA_DEBUG_SPIN_LIMIT = 0 makes
+    every merge go ahead without waiting, so every kernel still ends normally."""
+    from flash_attention_factory_amd import _cabi
+    w = W.make_config(1, num_seqs=4, pool_blocks=512)
+    try:
+        os.environ["FA_DEBUG_SPIN_LIMIT"] = "0"
+        for kernel in ("loop", "reduce"):
+            with pytest.raises(_cabi.PagedAttentionError, match="gave up waiting") as e:
+                for _ in range(20):  # whether a wavefront finds the others' states missing is a matter of timing
+                    _run(w, kernel)
+            assert e.value.code == _cabi.FA_ERR_RUNTIME
+    finally:
+        del os.environ["FA_DEBUG_SPIN_LIMIT"]
+    for kernel in ("loop", "reduce"):  # the word was cleared with the report
+        bufs, _ = _run(w, kernel)
+        _check(bufs.out, w, oracle, f"{w.name}/{kernel} after the report")

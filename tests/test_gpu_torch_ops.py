@@ -170,3 +170,24 @@ def test_operators_with_modifiers_query_tokens_and_block_scales(oracle):
         graph.replay()
         torch.cuda.synchronize()
         check(qn, f"replay {it}")
+
+
+def test_reduce_operators_report_scratch_overflow_when_told_the_longest_context():
+    """exp_sums.size(-1) partitions must cover the longest context; with max_context_len the operators
+    fail instead of attending over a truncated context."""
+    from flash_attention_factory_amd import _cabi, torch_ops  # noqa: F401
+    dev = _dev()
+    ops = torch.ops.fa_amd
+    for index in (0, 3):
+        w = W.make_config(index, num_seqs=2, pool_blocks=300, lens=[1300, 40]).to(dev)
+        kv, vv = _views(w, w.key_cache, w.value_cache)
+        bufs = runner.alloc_buffers(w, max_num_partitions=2)  # 2 x 512 tokens < 1300
+        args = (bufs.out, bufs.exp_sums, bufs.max_logits, bufs.tmp_out, w.query, kv, vv, w.block_tables, w.context_lens,
+                w.scale) + ((w.fp8_scale,) if w.is_fp8 else ()) + (512,)
+        op = ops.paged_attention_fp8_reduce if w.is_fp8 else ops.paged_attention_reduce
+        with pytest.raises(_cabi.PagedAttentionError, match="partitions"):
+            op(*args, max_context_len=1300)
+        fits = runner.alloc_buffers(w, max_num_partitions=3)
+        op(fits.out, fits.exp_sums, fits.max_logits, fits.tmp_out, *args[4:], max_context_len=1300)
+        torch.cuda.synchronize()
+        assert torch.isfinite(fits.out.float()).all()
