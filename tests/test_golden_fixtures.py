@@ -10,6 +10,8 @@ import numpy as np
 import pytest
 import torch
 
+from _torch_ref import assert_close_to_reference
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(HERE, "golden", "make_fixtures.py"))
 mk = importlib.util.module_from_spec(spec)
@@ -50,7 +52,7 @@ def test_kernels_match_fixtures(golden, name):
         bufs = runner.alloc_buffers(w)
         runner.run_workload(w, kernel, bufs)
         torch.cuda.synchronize()
-        torch.testing.assert_close(bufs.out.float().cpu(), want, atol=1e-2, rtol=1e-2)
+        assert_close_to_reference(bufs.out, want, f"{name}/{kernel}")
         if "reduce" in kernel:
             live = ~np.isnan(golden[f"{name}/exp_sums"])
             np.testing.assert_allclose(bufs.max_logits.cpu().numpy()[live], golden[f"{name}/max_logits"][live],

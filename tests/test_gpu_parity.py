@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from flash_attention_factory_amd import workloads as W
-from _torch_ref import call_oracle
+from _torch_ref import call_oracle, out_pt_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -32,7 +32,7 @@ def _run(w_cpu, kernel, max_context_len=None, schedule=0, **kw):
     return bufs, times
 
 
-def _check(out, w_cpu, oracle, label):
+def _check(out, w_cpu, oracle, label, literal_rule=False):
     ref16, ref32 = call_oracle(oracle.attention_ref, w_cpu, want_f32=True)
     got = out.float().cpu()
     err = (got - ref32).abs().max().item()
@@ -45,6 +45,13 @@ def _check(out, w_cpu, oracle, label):
     ulp = 2.0 ** (-8 if w_cpu.query.dtype == torch.bfloat16 else -11) * mag
     bar = 3 * max((model32 - ref32).abs().max().item(), ulp) + 1e-5
     assert err <= bar, f"{label}: err {err:.3e} above relative bar {bar:.3e}"
+    if literal_rule:
+        # upstream's own assertion, word for word (test_paged.py:603-604): both errors against the
+        # upcast reference rounded to the 16-bit type
+        live = w_cpu.context_lens > 0
+        err16 = (out.cpu()[live].float() - ref16[live].float()).abs().max().item()
+        err_pt = (out_pt_reference(w_cpu)[live].float() - ref16[live].float()).abs().max().item()
+        assert err16 <= 3 * err_pt + 1e-5, f"{label}: err {err16:.3e} above upstream's 3 x {err_pt:.3e} + 1e-5"
 
 
 SMALL = {  # measured configurations cut down so the oracle finishes in seconds
@@ -402,6 +409,76 @@ def test_e4m3_special_bytes(oracle):
     torch.testing.assert_close(got, ref, atol=5e-2, rtol=1e-2)    # values up to 448: the bar scales with them
 
 
+@pytest.mark.parametrize("qdtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", [W.TOKEN_MAJOR, W.HEAD_MAJOR])
+def test_e5m2_special_bytes(oracle, qdtype, layout):
+    """Every E5M2 byte through the decode of both FP8 kernels (fp16 queries: the byte-permute decode;
+    bf16 queries: the CDNA4 conversion instruction): all 248 finite codes -- both zeros, the
+    subnormals, up to +-57344 -- as K and V values inside the contexts, the infinity and NaN codes
+    in every row past a context's end."""
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    finite = codes[(codes & 0x7c) != 0x7c]
+    special = codes[(codes & 0x7c) == 0x7c]  # +-inf and the six NaN codes
+    assert finite.numel() == 248 and special.numel() == 8
+    g = torch.Generator().manual_seed(1)
+    w = W.make_test_shaped(batch_size=3, nheads=8, nheads_k=2, d=128, seqlen_k=640, varlen=False, has_sinks=False,
+                           fp8=True, block_size=16, dtype=qdtype, layout=layout)
+    w.context_lens = torch.tensor([640, 333, 17], dtype=torch.int32)
+    n = w.key_cache.numel()
+    kb, vb = w.key_cache.view(torch.uint8), w.value_cache.view(torch.uint8)
+    kb.view(-1).copy_(finite[torch.randint(0, 248, (n,), generator=g)])
+    vb.view(-1).copy_(finite[torch.randint(0, 248, (n,), generator=g)])
+    B = w.block_size
+    for s_ in range(3):  # rows at and past the end of each context: infinities and NaNs
+        ctx = int(w.context_lens[s_])
+        for col in range(ctx // B, w.block_tables.shape[1]):
+            blk = int(w.block_tables[s_, col])
+            first = ctx - col * B if col == ctx // B else 0
+            rows = slice(max(first, 0), B)
+            for pool in (kb, vb):
+                view = pool[blk] if layout == W.TOKEN_MAJOR else pool[blk].permute(1, 0, 2)  # [row, head, d]
+                view[rows] = special[torch.randint(0, 8, tuple(view[rows].shape), generator=g)]
+    w.scale = 1e-6  # values reach 57344: keeps the logits moderate
+    ref = call_oracle(oracle.attention_ref, w, want_f32=True)[1]
+    assert torch.isfinite(ref).all()
+    unit = ref.abs().max()
+    for kernel in ("fp8_loop", "fp8_reduce"):
+        for schedule in (0, 1):
+            bufs, _ = _run(w, kernel, schedule=schedule)
+            got = bufs.out.float().cpu()
+            assert torch.isfinite(got).all(), (kernel, schedule)
+            torch.testing.assert_close(got / unit, ref / unit, atol=ATOL, rtol=RTOL,
+                                       msg=lambda m: f"{kernel} schedule {schedule}: {m}")
+
+
+@pytest.mark.parametrize("qdtype", [torch.float16, torch.bfloat16])
+def test_e5m2_infinities_inside_the_context(oracle, qdtype):
+    """+-inf bytes among the values a query sees act as IEEE arithmetic says, in the kernels as in the
+    oracle: an infinite V entry under uniform weights makes that output element infinite (NaN where
+    both signs meet), an infinite K row makes the rows of its sequence NaN; other sequences are untouched."""
+    w = W.make_test_shaped(batch_size=3, nheads=4, nheads_k=2, d=128, seqlen_k=96, varlen=False, has_sinks=False,
+                           fp8=True, block_size=16, dtype=qdtype)
+    w.query[0] = 0                      # sequence 0: uniform weights
+    w.query[1] = w.query[1].abs() + 0.5  # sequence 1: positive queries, so an all-+inf K row scores +inf
+    kb, vb = w.key_cache.view(torch.uint8), w.value_cache.view(torch.uint8)
+    b0, b1 = int(w.block_tables[0, 2]), int(w.block_tables[1, 1])
+    vb[b0, 3, 0, 5] = 0x7c     # +inf: token 35 of sequence 0, kv head 0, d 5
+    vb[b0, 4, 0, 9] = 0xfc     # -inf: d 9
+    vb[b0, 5, 1, 7] = 0x7c     # kv head 1: +inf and -inf in the same column -> NaN
+    vb[b0, 6, 1, 7] = 0xfc
+    kb[b1, 2, 0, :] = 0x7c     # sequence 1, token 18, kv head 0: a K row of +inf
+    ref = call_oracle(oracle.attention_ref, w, want_f32=True)[1]
+    assert torch.isposinf(ref[0, 0, 5]) and torch.isneginf(ref[0, 1, 9]) and torch.isnan(ref[0, 2, 7])
+    assert torch.isnan(ref[1, :2]).all() and torch.isfinite(ref[1, 2:]).all() and torch.isfinite(ref[2]).all()
+    for kernel in ("fp8_loop", "fp8_reduce"):
+        bufs, _ = _run(w, kernel)
+        got = bufs.out.float().cpu()
+        assert torch.equal(torch.isnan(got), torch.isnan(ref)), kernel
+        assert torch.equal(torch.isposinf(got), torch.isposinf(ref)) and torch.equal(torch.isneginf(got), torch.isneginf(ref)), kernel
+        fin = torch.isfinite(ref)
+        torch.testing.assert_close(got[fin], ref[fin], atol=ATOL, rtol=RTOL)
+
+
 def test_bf16_and_fp8_scale(oracle):
     # bf16 queries with a bf16 cache, and with an FP8 cache at a non-unit scale
     w = W.make_test_shaped(batch_size=2, nheads=8, nheads_k=2, d=128, seqlen_k=700, varlen=True,
@@ -427,7 +504,9 @@ def test_whole_upstream_grid(oracle, heads, fp8):
     """Every case of the upstream test grid (test_paged.py:211-256, test_paged_fp8cache.py:220-264:
     batch 1/2 x sinks x var-len x head size 128/64 x nine head pairs x ten context lengths, block
     64, fp16) through the loop and the split kernel, with upstream's own gate next to the
-    absolute one (err <= 3 x err of the rounding-faithful model + 1e-5, test_paged.py:603-604).
+    absolute one, twice: err <= 3 x err of the rounding-faithful kernel model + 1e-5, and literally,
+    err <= 3 x err(out_pt) + 1e-5 with out_pt the reference evaluated without the fp32 upcast
+    (test_paged.py:432-447, 603-604).
     The seven lengths up to 2048 in full; of the three long ones (20000-50000) one combination of
     the other parameters each, rotating -- the oracle needs a third of a second for those -- unless
     FA_FULL_UPSTREAM_GRID=1 asks for all 2 x 1440 cases."""
@@ -440,7 +519,7 @@ def test_whole_upstream_grid(oracle, heads, fp8):
                                    has_sinks=s, fp8=fp8)
             for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
                 bufs, _ = _run(w, kernel)
-                _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
+                _check(bufs.out, w, oracle, f"{w.name}/{kernel}", literal_rule=True)
             n += 1
     everything = os.environ.get("FA_FULL_UPSTREAM_GRID") == "1"   # the long lengths in full too: minutes
     for k, seqlen_k in enumerate(UPSTREAM_LONG):
@@ -450,7 +529,7 @@ def test_whole_upstream_grid(oracle, heads, fp8):
                                    has_sinks=s, fp8=fp8)
             for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
                 bufs, _ = _run(w, kernel)
-                _check(bufs.out, w, oracle, f"{w.name}/{kernel}")
+                _check(bufs.out, w, oracle, f"{w.name}/{kernel}", literal_rule=True)
             n += 1
     assert n == len(UPSTREAM_SHORT) * 16 + len(UPSTREAM_LONG) * (16 if everything else 1)
 
