@@ -12,8 +12,19 @@ value        algorithmic bytes per step / wall time per step over K asynchronous
 roofline     per-kernel HIP-event time on the launch stream (the library's own
              elapsed_us path), HBM-bound
 cpu_baseline the CPU oracle (C + OpenMP restatement of the upstream tests' PyTorch
-             reference) on the same workload on this box's host cores
-configs      the other four configurations, each timed the same way
+             reference) on the same workload on this box's host cores; under "torch_reference"
+             that reference itself, restated in PyTorch (oracle/torch_reference.py), on a bounded
+             sample of every configuration: one sequence and kv head at a time, and for
+             configurations 0, 1 and 3 also in its literal padded form
+configs      the other four configurations, each timed the same way, each with a roofline block
+             of its own; the split configurations also say how many partitions one partial
+             covers, how many scratch bytes were really written, and carry a "strict_partitions"
+             leg: upstream's decomposition, one partial per 512-token partition
+reference_perf_recipe  the shape upstream's own perf loop runs (test_paged.py:607-631 and the FP8
+             twin: 64 sequences of 1500 tokens, 64 or 40 query heads over 8 kv heads, head size 64,
+             block size 64, sinks, its token-major pools) through the loop and the split kernels,
+             with upstream's bandwidth figure (bytes of the whole pool, test_paged.py:524-526)
+             beside the algorithmic one
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
 query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step);
              query_tokens_two_tiles: with 32, which fill two tiles of MFMA columns
@@ -44,10 +55,26 @@ HBM_PEAK_GBPS = 8000.0
 # 512-sequence variants of the configurations (--large-batches): blocks per pool
 LARGE_BATCH_POOL_BLOCKS = {1: 49152, 3: 49152, 4: 220000}
 
-MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE + WRITE_SIZE of paged_attn_loop_persistent_kernel<128, F16, kv16> per launch,
-    # profiles/paged_attn_kernels_bench_configs.md
-    "config1_loop": 661.20e6 + 0.26e6,
+def _measured_traffic():
+    """HBM bytes per launch of each configuration's dominant kernel, from the rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE runs summarised in profiles/hbm_traffic.txt (lines: name fetch_MB
+    write_MB).  None for a configuration the file does not list."""
+    table = {}
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if os.path.exists(path):
+        for line in open(path):
+            parts = line.split()
+            if len(parts) >= 3 and not line.startswith("#"):
+                table[parts[0]] = (float(parts[1]) + float(parts[2])) * 1e6
+    return table
+
+
+KERNEL_NAMES = {
+    0: "paged_attn_loop_persistent_kernel<64, F16, kv16, 4 waves>",
+    1: "paged_attn_loop_persistent_kernel<128, F16, kv16, 4 waves>",
+    2: "paged_attn_segment_kernel<128, F16, kv16, 4 waves>",
+    3: "paged_attn_loop_persistent_kernel<128, F16, e5m2, 4 waves>",
+    4: "paged_attn_segment_kernel<128, BF16, e5m2, 4 waves>",
 }
 
 
@@ -65,29 +92,28 @@ def _build_config(index, torch, W, runner, dev, **kw):
     return w, ks, vs
 
 
-def _time_config(built, steps, warmup, torch, W, runner, dev):
+def _time_config(built, steps, warmup, torch, W, runner, dev, schedule=0, traffic_key=None):
     w, ks, vs = built
-    kernel = W.CONFIG_KERNEL[w.meta["config"]]
+    kernel = W.CONFIG_KERNEL[w.meta["config"]] if "config" in w.meta else w.meta["kernel"]
     bufs = runner.alloc_buffers(w)
     n = len(ks)
     for it in range(warmup):
-        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False)
+        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False, schedule=schedule)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for it in range(steps):
-        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False)
+        runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], timed=False, schedule=schedule)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     # per-kernel durations from HIP events on the launch stream
     ev = []
     for it in range(steps):
-        ev.append(runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n]))
+        ev.append(runner.run_workload(w, kernel, bufs, key_cache=ks[it % n], value_cache=vs[it % n], schedule=schedule))
     ev_t = torch.tensor(ev, dtype=torch.float64)
     res = dict(
         workload=w.name, kernel=kernel, steps=steps,
         ms_per_step=wall / steps * 1e3,
         algorithmic_bytes=w.algorithmic_bytes(),
-        scratch_bytes=w.scratch_bytes() if "reduce" in kernel else 0,
         kernel_us_mean=[float(x) for x in ev_t.mean(0)],
         kernel_us_median=[float(x) for x in ev_t.median(0).values],
         us_per_call=float(ev_t.sum(1).mean()),
@@ -97,11 +123,32 @@ def _time_config(built, steps, warmup, torch, W, runner, dev):
     res["gbps_kernels"] = res["algorithmic_bytes"] / (res["us_per_call"] * 1e-6) / 1e9
     res["hbm_frac"] = res["gbps_kernels"] / HBM_PEAK_GBPS
     # the dominant kernel alone (the attention kernel; the reduce kernel is reported beside it)
-    res["gbps_attention_kernel"] = res["algorithmic_bytes"] / (res["kernel_us_mean"][0] * 1e-6) / 1e9
+    kernel_us = res["kernel_us_mean"][0]
+    achieved = res["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9
+    res["gbps_attention_kernel"] = achieved
+    res["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": achieved / HBM_PEAK_GBPS, "traffic": _measured_traffic().get(traffic_key),
+                       "kernel": KERNEL_NAMES.get(w.meta.get("config")) if schedule == 0 else "paged_attn_kernel (grid form)",
+                       "kernel_us": kernel_us}
+    if "reduce" in kernel:
+        # What the attention kernel really leaves in the scratch arrays: one call into NaN-filled
+        # buffers, then count.  A partial is (head_size + 2) floats per query head.
+        probe = runner.alloc_buffers(w)
+        runner.run_workload(w, kernel, probe, timed=False, schedule=schedule)
+        torch.cuda.synchronize()
+        written = ~torch.isnan(probe.max_logits)
+        S, H, D = w.query.shape
+        longest = int(torch.argmax(w.context_lens))
+        slots = torch.nonzero(written[longest, 0]).flatten().tolist()
+        res["scratch_bytes_allocated"] = w.scratch_bytes()
+        res["scratch_bytes_written"] = int(written.sum()) * (D + 2) * 4
+        res["partials"] = int(written.sum()) // H * w.num_kv_heads
+        res["partitions_per_segment"] = (slots[1] - slots[0]) if len(slots) > 1 else None
+        res["partition_size"] = w.partition_size
     return w, res
 
 
-def _cpu_baseline(index, torch, W, budget_s=12.0):
+def _cpu_baseline(index, torch, W, budget_s=10.0):
     from oracle import oracle as O
     w = W.make_config(index)  # CPU generator, seeded
     def call():
@@ -121,6 +168,76 @@ def _cpu_baseline(index, torch, W, budget_s=12.0):
                 ms_per_call=per * 1e3,
                 sample=f"full {w.name} workload (seed 0), {reps} repetitions of the C/OpenMP oracle "
                        f"oracle_attention_ref, {dt:.1f} s")
+
+
+# Bounded samples of the configurations for the PyTorch reference on the host cores: the same
+# shapes and length distributions with fewer sequences (and pools just large enough for them),
+# so that the whole leg stays within seconds.
+_TORCH_SAMPLES = {0: dict(), 1: dict(), 2: dict(num_seqs=2, pool_blocks=4096), 3: dict(),
+                  4: dict(num_seqs=16, pool_blocks=12288)}
+
+
+def _torch_reference_baseline(torch, W, budget_s=2.5):
+    """The upstream tests' PyTorch reference (oracle/torch_reference.py) timed on this box's host
+    cores with torch's own threading: per configuration the per-sequence form, and for
+    configurations 0, 1 and 3 also the literal padded form (dense K/V gathered and repeated over
+    the query group, as test_paged.py builds them)."""
+    from oracle import torch_reference as T
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    out = []
+    for index, kw in _TORCH_SAMPLES.items():
+        w = W.make_config(index, **kw)
+        forms = [("per_sequence", False)] + ([("padded", True)] if index in (0, 1, 3) else [])
+        for form, padded in forms:
+            T.run_workload(w, padded=padded)  # warm-up
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                T.run_workload(w, padded=padded)
+                reps += 1
+                dt = time.perf_counter() - t0
+                if dt > budget_s or reps >= 50:
+                    break
+            per = dt / reps
+            full = W._CONFIGS[index]["S"]
+            out.append(dict(config=index, form=form, value=w.algorithmic_bytes() / per / 1e9, unit="GB/s",
+                            ms_per_call=per * 1e3, cores=threads, torch_threads=torch.get_num_threads(), kind="port",
+                            sample=f"{w.num_seqs} of the {full} sequences of {w.name} "
+                                   f"({w.algorithmic_bytes() / 1e6:.1f} MB of K/V), {reps} repetitions, {dt:.1f} s"
+                                   + (f", dense K/V of {T.padded_bytes(w) / 1e6:.0f} MB" if padded else "")))
+    return out
+
+
+def _reference_perf_recipe(steps, torch, W, runner, dev):
+    """Upstream's own perf shape and loop (test_paged.py:607-631, 485-560; FP8 twin
+    test_paged_fp8cache.py:612-636): batch 64, 64 (FP8: 40) query heads over 8 kv heads, 1500 keys,
+    head size 64, block size 64, sinks, pools in upstream's token-major layout with every block
+    referenced by exactly one sequence, several pool clones rotated, 5 warm-up calls, kernel-event
+    time.  Upstream counts the bytes of the whole pool (:524-526); the algorithmic figure (keys
+    inside the contexts only) is given beside it."""
+    legs = []
+    for fp8, heads in ((False, 64), (True, 40)):
+        w = W.make_test_shaped(batch_size=64, nheads=heads, nheads_k=8, d=64, seqlen_k=1500, varlen=False,
+                               has_sinks=True, fp8=fp8, device=dev)
+        w.meta["kernel"] = "fp8_loop" if fp8 else "loop"
+        pool_bytes = w.key_cache.numel() * w.key_cache.element_size() * 2
+        ks, vs = _clones(w, torch)
+        for kernel in ((("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce"))):
+            bufs = runner.alloc_buffers(w)
+            ts = []
+            for it in range(5 + steps):
+                t = runner.run_workload(w, kernel, bufs, key_cache=ks[it % len(ks)], value_cache=vs[it % len(ks)])
+                if it >= 5:
+                    ts.append(sum(t))
+            us = float(torch.tensor(ts, dtype=torch.float64).mean())
+            legs.append(dict(workload=f"upstream perf recipe: S64 H{heads} Hk8 D64 B64 ctx1500 sinks, token-major, "
+                                      f"{'E5M2' if fp8 else 'fp16'} pools", kernel=kernel, steps=steps,
+                             us_per_call=us, pool_clones=len(ks), whole_pool_bytes=pool_bytes,
+                             gbps_whole_pool=pool_bytes / us / 1e3,
+                             algorithmic_bytes=w.algorithmic_bytes(), gbps_kernels=w.algorithmic_bytes() / us / 1e3,
+                             hbm_frac=w.algorithmic_bytes() / us / 1e3 / HBM_PEAK_GBPS))
+        del ks, vs, w
+    return legs
 
 
 def _time_kv_cache_write(steps, torch, dev, cpu_leg):
@@ -352,14 +469,19 @@ def main():
     built = {i: _build_config(i, torch, W, runner, dev, layout=args.layout) for i in order}
     torch.cuda.synchronize()
 
-    _, main_res = _time_config(built[1], args.steps, args.warmup, torch, W, runner, dev)
+    _, main_res = _time_config(built[1], args.steps, args.warmup, torch, W, runner, dev,
+                               traffic_key="config1" + ("" if args.layout == "head_major" else "_token_major"))
     others = []
+    sub_steps = max(20, args.steps // 2)
+    suffix = "" if args.layout == "head_major" else "_token_major"
     for idx in indices[1:]:
-        _, r = _time_config(built[idx], max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+        _, r = _time_config(built[idx], sub_steps, args.warmup, torch, W, runner, dev, traffic_key=f"config{idx}{suffix}")
+        if "reduce" in r["kernel"] and not args.no_extras:
+            # upstream's own decomposition: one work-group and one partial per 512-token partition
+            _, strict = _time_config(built[idx], sub_steps, args.warmup, torch, W, runner, dev, schedule=1)
+            r["strict_partitions"] = {k: strict[k] for k in ("kernel_us_mean", "us_per_call", "gbps_kernels", "hbm_frac",
+                                                            "scratch_bytes_written", "partials", "partitions_per_segment")}
         others.append(r)
-
-    kernel_us = main_res["kernel_us_mean"][0]
-    achieved = main_res["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9
     line = {
         "metric": "achieved HBM GB/s, fp16 paged decode (loop kernel)",
         "value": main_res["gbps_wall"],
@@ -375,14 +497,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config1: fp16 loop kernel, S32 H32 Hk32 D128 B16 ctx U[512,2048], "
                                "4096-block head-major pool, shuffled block tables",
+                   "layout": args.layout,
                    "us_per_call": main_res["us_per_call"],
                    "algorithmic_bytes": main_res["algorithmic_bytes"],
                    "hbm_frac_of_8TBps": main_res["hbm_frac"]},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("config1_loop"),
-                     "kernel": "paged_attn_loop_persistent_kernel<128, F16, kv16, 4 waves>",
-                     "kernel_us": kernel_us},
+        "roofline": main_res.pop("roofline"),
         "configs": others,
     }
     if not args.no_extras:
@@ -402,12 +521,15 @@ def main():
         # [blocks, block_size, kv_heads, head_size]: a token's row of one kv head is then the only
         # contiguous piece (256 or 128 bytes), successive tokens lie kv_heads rows apart
         line["token_major_layout"] = []
-        for idx in (() if args.no_token_major else (1, 3)):
+        for idx in (() if args.no_token_major else (4, 2, 1, 3)):
             tm = _build_config(idx, torch, W, runner, dev, layout=W.TOKEN_MAJOR)
-            _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
+            _, r = _time_config(tm, max(20, args.steps // 2), args.warmup, torch, W, runner, dev,
+                                traffic_key=f"config{idx}_token_major")
             r["workload"] += "_token_major"
             line["token_major_layout"].append(r)
             del tm
+        line["token_major_layout"].sort(key=lambda r: r["workload"])
+        line["reference_perf_recipe"] = _reference_perf_recipe(max(20, args.steps // 2), torch, W, runner, dev)
         line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
         del built
@@ -415,6 +537,7 @@ def main():
         line["kv_cache_write"] = _time_kv_cache_write(max(20, args.steps // 2), torch, dev, not args.no_cpu_baseline)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(1, torch, W)
+        line["cpu_baseline"]["torch_reference"] = _torch_reference_baseline(torch, W)
     if args.large_batches:
         # Pools of tens of GB want an allocator nobody has fragmented (see above): one child
         # process per configuration, after this process has given its own pools back.
