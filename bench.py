@@ -20,6 +20,8 @@ configs      the other four configurations, each timed the same way, each with a
              of its own; the split configurations also say how many partitions one partial
              covers, how many scratch bytes were really written, and carry a "strict_partitions"
              leg: upstream's decomposition, one partial per 512-token partition
+lds_staging  the FP8 configurations in the grid form, K/V through registers against K/V staged
+             through LDS by direct-to-LDS loads
 reference_perf_recipe  the shape upstream's own perf loop runs (test_paged.py:607-631 and the FP8
              twin: 64 sequences of 1500 tokens, 64 or 40 query heads over 8 kv heads, head size 64,
              block size 64, sinks, its token-major pools) through the loop and the split kernels,
@@ -529,6 +531,16 @@ def main():
             line["token_major_layout"].append(r)
             del tm
         line["token_major_layout"].sort(key=lambda r: r["workload"])
+        # the grid form of the FP8 configurations with K/V through registers (schedule 1) and staged
+        # through LDS by direct-to-LDS loads (schedule 2), beside the persistent forms timed above
+        line["lds_staging"] = []
+        for idx in (3, 4):
+            if idx not in built:
+                continue
+            for schedule, name in ((1, "grid form, K/V through registers"), (2, "grid form, K/V staged through LDS")):
+                _, r = _time_config(built[idx], sub_steps, args.warmup, torch, W, runner, dev, schedule=schedule)
+                line["lds_staging"].append(dict(workload=r["workload"], schedule=name, kernel_us_mean=r["kernel_us_mean"],
+                                                us_per_call=r["us_per_call"], hbm_frac=r["hbm_frac"]))
         line["reference_perf_recipe"] = _reference_perf_recipe(max(20, args.steps // 2), torch, W, runner, dev)
         line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:
