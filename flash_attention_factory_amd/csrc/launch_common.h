@@ -230,9 +230,13 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
 // do not look: the word stays set until the next timed call on the device reports it.
 inline fa_status report_kernel_status(const Resolved &r) {
   if (!r.elapsed_us || !r.status) return FA_OK;
-  int32_t seen = 0;
-  FA_HIP_CHECK(hipMemcpyAsync(&seen, r.status, sizeof(seen), hipMemcpyDeviceToHost, r.stream));
+  // read through one pinned word per thread (a copy into pageable memory costs ten times as much);
+  // allocated on the first timed call, like the timing events
+  static thread_local int32_t *pinned = nullptr;
+  if (pinned == nullptr) FA_HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&pinned), sizeof(int32_t), hipHostMallocDefault));
+  FA_HIP_CHECK(hipMemcpyAsync(pinned, r.status, sizeof(int32_t), hipMemcpyDeviceToHost, r.stream));
   FA_HIP_CHECK(hipStreamSynchronize(r.stream));
+  const int32_t seen = *pinned;
   if (seen == 0) return FA_OK;
   const int32_t zero = 0;
   FA_HIP_CHECK(hipMemcpyAsync(r.status, &zero, sizeof(zero), hipMemcpyHostToDevice, r.stream));
