@@ -107,6 +107,7 @@ struct Resolved {
   const float *k_scales;
   const float *v_scales;
   int32_t schedule;  // fa_schedule
+  bool pair_heads;   // two adjacent kv heads with 64-byte token rows run as one (WaveAttn::kPairable)
   int32_t *status;   // status word of the current device (nullptr with validate_only)
   int32_t spin_limit;
   hipStream_t stream;
@@ -215,6 +216,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->schedule = o ? o->schedule : FA_SCHEDULE_AUTO;
   if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS)
     return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2)", r->schedule);
+  r->pair_heads = kPairHeads && kv8 && s->head_size == 64 && s->kv_head_stride == s->head_size &&
+                  s->num_kv_heads % 2 == 0 && 2 * r->group <= kMaxGroup && r->mask_flags == 0 &&
+                  r->query_len == 1 && r->kv_scale_mode == FA_KV_SCALE_TENSOR;
   r->stream = o ? reinterpret_cast<hipStream_t>(o->stream) : nullptr;
   r->elapsed_us = o ? o->elapsed_us : nullptr;
   r->validate_only = o && o->validate_only != 0;
@@ -287,6 +291,13 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.kv_block_bytes = s.kv_block_stride * r.kv_elem_bytes;
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;
+  p.pair_heads = 0;
+  if (r.pair_heads) {  // the kernel sees pairs of kv heads: half as many, twice the group, rows of two heads
+    p.pair_heads = 1;
+    p.num_kv_heads /= 2;
+    p.group *= 2;
+    p.kv_head_bytes *= 2;
+  }
   return p;
 }
 

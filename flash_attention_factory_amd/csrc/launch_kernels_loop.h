@@ -28,7 +28,7 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
   PagedAttnParams p = make_params(out, nullptr, nullptr, query, key_cache, value_cache,
                                   block_tables, context_lens, scale, shape, r);
   KernelTimer timer(r.elapsed_us != nullptr, r.stream);
-  const int64_t items = (int64_t)shape.num_seqs * shape.num_kv_heads;
+  const int64_t items = (int64_t)shape.num_seqs * p.num_kv_heads;  // pairs of kv heads with r.pair_heads
   const int64_t max_ctx = (int64_t)shape.max_blocks_per_seq * shape.block_size;
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
@@ -58,20 +58,20 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
       const dim3 grid((unsigned)std::min<int64_t>(resident, items));
       FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
-    } else if (KV8 && HEAD_SIZE == 128 && !ext && r.schedule == FA_SCHEDULE_GRID_LDS) {
+    } else if (KV8 && HEAD_SIZE == 128 && !ext && !r.pair_heads && r.schedule == FA_SCHEDULE_GRID_LDS) {
       // grid form, K and V staged through LDS: one work-group of eight wavefronts per compute unit
       if constexpr (KV8 && HEAD_SIZE == 128) {
-        const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+        const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);
         FA_HIP_CHECK(timer.launch(paged_attn_lds_kernel<HEAD_SIZE, QT, KVF, false, 8, 2>, grid, dim3(8 * 64), 0, p));
       }
     } else if (ext) {
-      const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+      const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
                             Pipeline<KV8>::tiles_per_chunk, true, KROW>,
           grid, dim3(NW * 64), 0, p));
     } else {
-      const dim3 grid(shape.num_kv_heads, 1, shape.num_seqs);
+      const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, false, NW, Pipeline<KV8>::occ,
                             Pipeline<KV8>::tiles_per_chunk, false, KROW>,
@@ -91,6 +91,11 @@ inline fa_status launch_paged_attn_loop_batch(void *out, const void *query, cons
                                               const int32_t *context_lens, float scale,
                                               const fa_paged_attention_shape &shape, const Resolved &r,
                                               float *total_us_out) {
+  if constexpr (KVF != kKv16 && HEAD_SIZE == 64) {
+    if (r.pair_heads)  // pairs of kv heads as rows of 128 bytes: the head-size-128 instance
+      return launch_paged_attn_loop_rows<128, QT, KVF, true>(out, query, key_cache, value_cache, block_tables,
+                                                             context_lens, scale, shape, r, total_us_out);
+  }
   if constexpr (KVF == kKv16 && !kRowLoadsLoop16Adjacent) {
     if (shape.kv_token_stride == shape.head_size)
       return launch_paged_attn_loop_rows<HEAD_SIZE, QT, KVF, false>(out, query, key_cache, value_cache, block_tables,

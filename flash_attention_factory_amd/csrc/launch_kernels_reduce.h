@@ -18,7 +18,9 @@ namespace fa {
 // Attention and reduce launches of one batch that a single attention launch can take (segment
 // form for up to kSegmentMaxSeqs sequences, else the grid form).  Kernel times are ADDED to
 // us_out[0] (attention) and us_out[1] (reduce) when the call is timed.
-template <int HEAD_SIZE, typename QT, int KVF>
+// HEAD_SIZE: head size of the attention kernel instance; OUT_D: elements of a row of out and
+// tmp_out -- the same, except for pairs of kv heads (Resolved::pair_heads: 128 and 64).
+template <int HEAD_SIZE, typename QT, int KVF, int OUT_D = HEAD_SIZE>
 inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const void *key_cache,
                                             const void *value_cache, const int32_t *block_tables,
                                             const int32_t *context_lens, float scale,
@@ -70,24 +72,24 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
           resident = std::min(resident, other);
         }
         const int64_t max_items =
-            (int64_t)shape.num_seqs * shape.max_num_partitions * shape.num_kv_heads;
+            (int64_t)shape.num_seqs * shape.max_num_partitions * p.num_kv_heads;
         segment_groups = (int)std::min<int64_t>(resident, max_items);
       }
       FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
-    } else if (KV8 && HEAD_SIZE == 128 && !ext && r.schedule == FA_SCHEDULE_GRID_LDS) {
+    } else if (KV8 && HEAD_SIZE == 128 && !ext && !r.pair_heads && r.schedule == FA_SCHEDULE_GRID_LDS) {
       // grid form, K and V staged through LDS: one wavefront per partition
       if constexpr (KV8 && HEAD_SIZE == 128) {
-        const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+        const dim3 grid(p.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
         FA_HIP_CHECK(timer.launch(paged_attn_lds_kernel<HEAD_SIZE, QT, KVF, true, 1, 2>, grid, dim3(64), 0, p));
       }
     } else if (ext) {
-      const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+      const dim3 grid(p.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
                             Pipeline<KV8>::tiles_per_chunk, true>,
           grid, dim3(NW * 64), 0, p));
     } else {
-      const dim3 grid(shape.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
+      const dim3 grid(p.num_kv_heads, shape.max_num_partitions, shape.num_seqs);
       FA_HIP_CHECK(timer.launch(
           paged_attn_kernel<HEAD_SIZE, QT, KVF, true, NW, Pipeline<KV8>::occ,
                             Pipeline<KV8>::tiles_per_chunk>,
@@ -108,23 +110,43 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   rp.partition_size = r.partition_size;
   rp.max_context = (int32_t)std::min<int64_t>((int64_t)shape.max_blocks_per_seq * shape.block_size, INT32_MAX);
   rp.num_seqs = shape.num_seqs;
-  rp.num_kv_heads = shape.num_kv_heads;
+  rp.num_kv_heads = p.num_kv_heads;  // what the attention kernel dealt by: pairs with r.pair_heads
   rp.query_len = r.query_len;
   rp.segment_groups = segment_groups;
   const dim3 rgrid((unsigned)((int64_t)shape.num_heads * shape.num_seqs * r.query_len));
   const bool one_wave = (int64_t)shape.num_heads * shape.num_seqs * r.query_len >= kReduceSingleWaveMinPairs;
   if (segment_groups > 0) {
-    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, true>, rgrid, dim3(64), 1, rp));
-    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, true>, rgrid, dim3(256), 1, rp));
+    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<OUT_D, QT, 1, true>, rgrid, dim3(64), 1, rp));
+    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<OUT_D, QT, 4, true>, rgrid, dim3(256), 1, rp));
   } else {
-    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 1, false>, rgrid, dim3(64), 1, rp));
-    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<HEAD_SIZE, QT, 4, false>, rgrid, dim3(256), 1, rp));
+    if (one_wave) FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<OUT_D, QT, 1, false>, rgrid, dim3(64), 1, rp));
+    else FA_HIP_CHECK(timer.launch(paged_attn_reduce_kernel<OUT_D, QT, 4, false>, rgrid, dim3(256), 1, rp));
   }
   if (r.elapsed_us) {
     us_out[0] += attention_us;
     FA_HIP_CHECK(timer.accumulate(1, &us_out[1]));
   }
   return FA_OK;
+}
+
+// Pairs of kv heads (Resolved::pair_heads) run in the head-size-128 attention instance, everything
+// else in the instance of its own head size.
+template <int HEAD_SIZE, typename QT, int KVF>
+inline fa_status launch_paged_attn_v2_instance(void *out, const void *query, const void *key_cache,
+                                               const void *value_cache, const int32_t *block_tables,
+                                               const int32_t *context_lens, float scale,
+                                               float *exp_sums, float *max_logits, float *tmp_out,
+                                               const fa_paged_attention_shape &shape, const Resolved &r,
+                                               float *us_out) {
+  if constexpr (KVF != kKv16 && HEAD_SIZE == 64) {
+    if (r.pair_heads)
+      return launch_paged_attn_v2_batch<128, QT, KVF, 64>(out, query, key_cache, value_cache, block_tables,
+                                                          context_lens, scale, exp_sums, max_logits, tmp_out, shape,
+                                                          r, us_out);
+  }
+  return launch_paged_attn_v2_batch<HEAD_SIZE, QT, KVF>(out, query, key_cache, value_cache, block_tables,
+                                                        context_lens, scale, exp_sums, max_logits, tmp_out, shape, r,
+                                                        us_out);
 }
 
 // Whether the segment kernel takes batches of this shape at all (given few enough sequences).
@@ -161,14 +183,14 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
     for (int s0 = 0; s0 < shape.num_seqs; s0 += per) {
       fa_paged_attention_shape sub = shape;
       sub.num_seqs = std::min(per, shape.num_seqs - s0);
-      const fa_status st = launch_paged_attn_v2_batch<HEAD_SIZE, QT, KVF>(
+      const fa_status st = launch_paged_attn_v2_instance<HEAD_SIZE, QT, KVF>(
           reinterpret_cast<char *>(out) + s0 * row_bytes, reinterpret_cast<const char *>(query) + s0 * row_bytes,
           key_cache, value_cache, block_tables + (int64_t)s0 * shape.max_blocks_per_seq, context_lens + s0, scale,
           exp_sums + s0 * slots, max_logits + s0 * slots, tmp_out + s0 * slots * shape.head_size, sub, r, us);
       if (st != FA_OK) return st;
     }
   } else {
-    const fa_status st = launch_paged_attn_v2_batch<HEAD_SIZE, QT, KVF>(
+    const fa_status st = launch_paged_attn_v2_instance<HEAD_SIZE, QT, KVF>(
         out, query, key_cache, value_cache, block_tables, context_lens, scale, exp_sums, max_logits, tmp_out,
         shape, r, us);
     if (st != FA_OK) return st;

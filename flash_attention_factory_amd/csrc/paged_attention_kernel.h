@@ -72,22 +72,25 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
     }
   }
 
-  if (!wa.col_valid) return;
+  if (!wa.col_valid || !wa.keeps_output()) return;
   float out_scale = p.out_scale;
   if constexpr (W::kExt) out_scale = wa.out_mul;
   const float inv = L > 0.f ? out_scale / L : 0.f;  // L = 0: nothing visible (local window, causal rule)
   const int head = kvh * p.group + wa.col_g;
   const int64_t row = W::kExt ? (int64_t)seq * p.query_len + wa.col_q : seq;  // row of query / out / scratch
-  const int d0 = 4 * r * NDT + wave * SL;  // first head-dim element this lane stores
+  const int d0 = wa.out_elem(4 * r * NDT + wave * SL);  // first head-dim element this lane stores
+  const int DR = wa.out_row_elems();
   if constexpr (PART) {
     const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part;
-    W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
-    if (r == 0 && wave == 0) {
+    W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * DR + d0, o, inv);
+    // one lane per column writes the scalars: r = 0, or of the lanes that keep a paired column's
+    // output the first (r = 0 for the pair's first head, 2 for its second)
+    if ((wa.paired() ? (r & 1) == 0 : r == 0) && wave == 0) {
       p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
       p.exp_sums[slot] = L;
     }
   } else {
-    W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
+    W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * DR + d0) * 2, o, inv);
   }
 }
 

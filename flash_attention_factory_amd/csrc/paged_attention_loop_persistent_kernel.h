@@ -201,16 +201,17 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[tile][b][w][wave * SL + k][lane];
       o[k] = a;
     }
-    if (wa.col_valid) {
+    if (wa.col_valid && wa.keeps_output()) {
       const int head = kvh * p.group + wa.col_g;
-      const int d0 = 4 * r * NDT + wave * SL;
+      const int d0 = wa.out_elem(4 * r * NDT + wave * SL);
       int64_t row = seq;
       float inv = p.out_scale / L;
       if constexpr (EXT) {
         row = (int64_t)seq * p.query_len + wa.col_q;
         inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key
       }
-      W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
+      W::template store_q<SL>(
+          reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * wa.out_row_elems() + d0) * 2, o, inv);
     }
   };
 

@@ -69,6 +69,14 @@ struct WavesPerGroup {
 #endif
 constexpr bool kRowLoadsLoop16Adjacent = FA_K_ROW_LOADS_LOOP16_ADJACENT != 0;
 
+// FP8 caches with token rows of 64 bytes (head size 64) whose kv heads lie next to each other in
+// memory: take two kv heads as one row of 128 bytes (WaveAttn::kPairable).  Every cache line is
+// then fetched by one work-group instead of two.
+#ifndef FA_PAIR_HEADS
+#define FA_PAIR_HEADS 1
+#endif
+constexpr bool kPairHeads = FA_PAIR_HEADS != 0;
+
 template <bool kKV8>
 struct Pipeline {
   static constexpr int occ = kKV8 ? FA_OCC_FP8 : FA_OCC;

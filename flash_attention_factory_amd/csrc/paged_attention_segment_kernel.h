@@ -224,7 +224,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[tile][b][w][wave * SL + e][lane];
       o[e] = a;
     }
-    if (wa.col_valid) {
+    if (wa.col_valid && wa.keeps_output()) {
       const int head = it.kvh * p.group + wa.col_g;
       int64_t row = it.seq;
       float inv = p.out_scale / L;
@@ -233,9 +233,9 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
         inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key of the segment
       }
       const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
-      const int d0 = 4 * r * NDT + wave * SL;
-      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
-      if (r == 0 && wave == 0) {
+      const int d0 = wa.out_elem(4 * r * NDT + wave * SL);
+      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
+      if ((wa.paired() ? (r & 1) == 0 : r == 0) && wave == 0) {  // one lane per column, see merge_and_store
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;
       }

@@ -73,6 +73,11 @@ struct PagedAttnParams {
   // work-group before it gives up, and the device word in which it says so (see launch_common.h)
   int32_t spin_limit;
   int32_t *status;
+  // Paired kv heads (FP8 caches with token rows of 64 bytes whose kv heads lie next to each
+  // other): a head-size-128 instance takes two kv heads as one -- num_kv_heads, group and
+  // kv_head_bytes describe the pairs -- while query and out rows keep 64 elements.  See
+  // WaveAttn::kPairable.
+  int32_t pair_heads;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
@@ -109,6 +114,21 @@ struct WaveAttn {
   // 128 L + (i >> 3) * 64 + r * 16 for load c = 2L + h), and k_rows_to_mfma() moves the halves
   // that sit in the wrong lane across with DPP.  The head-dim <-> k-slot map stays what it was.
   static constexpr bool kRowLoads = FA_K_ROW_LOADS != 0 && KROW && ROWB >= 128;
+  // Paired kv heads (p.pair_heads).  With token rows of 64 bytes every 128-byte line of a
+  // token-major pool belongs to two kv heads; two work-groups would fetch it once each.  Here
+  // the two heads' rows are one 128-byte row of a pair: the 2G query heads of both are the MFMA
+  // columns, a column's query is zero over the other head's half of the row (so the scores are
+  // its own head's), and of the 128 output rows a column keeps the half that belongs to its
+  // head: lanes r = 0, 1 hold a pair's dims 0..63 (first head), r = 2, 3 dims 64..127 (second).
+  static constexpr bool kPairable = KV8 && D == 128 && !EXT;
+  __device__ __forceinline__ bool paired() const { return kPairable && p.pair_heads != 0; }
+  // which head of its pair column i belongs to
+  __device__ __forceinline__ int col_half() const { return i >= (p.group >> 1) ? 1 : 0; }
+  // does this lane hold output elements its column keeps, how long is a row of query / out /
+  // tmp_out, and which element of that row is the lane's first (d0: its first of the pair's 128)
+  __device__ __forceinline__ bool keeps_output() const { return !paired() || (r >> 1) == col_half(); }
+  __device__ __forceinline__ int out_row_elems() const { return paired() ? D / 2 : D; }
+  __device__ __forceinline__ int out_elem(int d0) const { return paired() ? d0 - (D / 2) * (r >> 1) : d0; }
 
 
   // Register image of one chunk of K and V.
@@ -229,12 +249,19 @@ struct WaveAttn {
   __device__ __forceinline__ void load_q(int seq, int kvh) {
     const int head = kvh * p.group + col_g;
     const int64_t row = EXT ? (int64_t)seq * p.query_len + col_q : seq;
-    const char *qrow = reinterpret_cast<const char *>(p.query) + (row * p.num_heads + head) * (D * 2);
+    const char *qrow = reinterpret_cast<const char *>(p.query) + (row * p.num_heads + head) * (out_row_elems() * 2);
 #pragma unroll
     for (int c = 0; c < KSTEPS; ++c) {
-      const int d0 = KV8 ? ((c >> 1) * 4 + r) * 16 + (c & 1) * 8 : (c * 4 + r) * 8;
+      int d0 = KV8 ? ((c >> 1) * 4 + r) * 16 + (c & 1) * 8 : (c * 4 + r) * 8;
+      bool live = col_valid;
+      if constexpr (kPairable) {
+        if (p.pair_heads) {  // k-steps 0, 1 run over the first head's dims, 2, 3 over the second's
+          live = live && (c >> 1) == col_half();
+          d0 -= (D / 2) * (c >> 1);
+        }
+      }
       u32x4 z = {0u, 0u, 0u, 0u};
-      qB[c] = col_valid ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
+      qB[c] = live ? *reinterpret_cast<const u32x4 *>(qrow + d0 * 2) : z;
     }
   }
 
