@@ -21,6 +21,7 @@
 #include "paged_attention_kernel.h"
 #include "paged_attention_lds_kernel.h"
 #include "paged_attention_loop_persistent_kernel.h"
+#include "paged_attention_loop_two_tile_kernel.h"
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
 #include "paged_attention_segment_kernel.h"

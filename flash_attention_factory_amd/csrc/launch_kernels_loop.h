@@ -37,7 +37,7 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
                           shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
                           max_ctx < kLoopPersistentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
-  // columns, or in the persistent form two tiles of 16 held by two halves of every work-group.
+  // columns, or in the persistent form two tiles of 16 held by every wavefront.
   const int per_tile = p.query_count;
   const int per_launch = (persistent && r.query_len > per_tile) ? 2 * per_tile : per_tile;
   for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {
@@ -51,8 +51,8 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
                                                      Pipeline<KV8>::tiles_per_chunk, false, 1, KROW>;
       auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
                                                         Pipeline<KV8>::tiles_per_chunk, true, 1, KROW>;
-      auto two_tiles = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                         Pipeline<KV8>::tiles_per_chunk, true, 2, KROW>;
+      // two column tiles in the registers of every wavefront: K and V are loaded once for both
+      auto two_tiles = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, PW, Pipeline<KV8>::tiles_per_chunk, KROW>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
       int resident = 0;
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));

@@ -506,6 +506,37 @@ struct WaveAttn {
         acc[dt] = mfma_16x16x32<QT>(v_operand(R, pr, dt), pb.v[pr], acc[dt]);
   }
 
+  // Two column tiles held by ONE wavefront (a and b: the same chunk, different 16 columns) share
+  // the K and V operands: every operand is built once and feeds both tiles' MFMAs.
+  static __device__ __forceinline__ void qk_two(const WaveAttn &a, const WaveAttn &b, Chunk &R, Scores &sa, Scores &sb) {
+    if constexpr (kRowLoads) {
+#pragma unroll
+      for (int t = 0; t < TPC; ++t)
+#pragma unroll
+        for (int c = 0; c < KL; c += 2) k_rows_to_mfma(R.k[t][c], R.k[t][c + 1]);
+    }
+#pragma unroll
+    for (int t = 0; t < TPC; ++t) sa.v[t] = sb.v[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KSTEPS; ++c)
+#pragma unroll
+      for (int t = 0; t < TPC; ++t) {
+        const u32x4 ko = a.k_operand(R, t, c);
+        sa.v[t] = mfma_16x16x32<QT>(ko, a.qB[c], sa.v[t]);
+        sb.v[t] = mfma_16x16x32<QT>(ko, b.qB[c], sb.v[t]);
+      }
+  }
+  static __device__ __forceinline__ void pv_two(WaveAttn &a, WaveAttn &b, const Chunk &R, const Probs &pa, const Probs &pb) {
+#pragma unroll
+    for (int pr = 0; pr < NP2; ++pr)
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const u32x4 vo = a.v_operand(R, pr, dt);
+        a.acc[dt] = mfma_16x16x32<QT>(vo, pa.v[pr], a.acc[dt]);
+        b.acc[dt] = mfma_16x16x32<QT>(vo, pb.v[pr], b.acc[dt]);
+      }
+  }
+
   // A lane's NR accumulator values are NR consecutive head-dim elements of head i:
   // d = 4r*NDT + idx with idx = e*NDT + dt.
   __device__ __forceinline__ float acc_at(int idx) const { return acc[idx % NDT][idx / NDT]; }

@@ -612,3 +612,33 @@ def test_exhausted_spin_limit_is_reported(oracle):
     for kernel in ("loop", "reduce"):  # the word was cleared with the report
         bufs, _ = _run(w, kernel)
         _check(bufs.out, w, oracle, f"{w.name}/{kernel} after the report")
+
+
+@pytest.mark.parametrize("heads", [(32, 4), (40, 8), (8, 8), (6, 2), (9, 3)], ids=lambda h: f"h{h[0]}x{h[1]}")
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_fp8_head_size_64_pairs_of_kv_heads(oracle, heads, block_size):
+    """FP8 caches with 64-byte token rows in upstream's token-major layout: two adjacent kv heads share
+    every cache line and run as one 128-byte row (several pairs per sequence, groups up to 8, an odd
+    number of kv heads that cannot pair, the head-major layout where heads are not adjacent) -- loop
+    and split, persistent and grid forms, scratch contents per partition under the grid form."""
+    nheads, nheads_k = heads
+    for layout in (W.TOKEN_MAJOR, W.HEAD_MAJOR):
+        w = W.make_test_shaped(batch_size=5, nheads=nheads, nheads_k=nheads_k, d=64, seqlen_k=900, varlen=False,
+                               has_sinks=False, fp8=True, block_size=block_size, layout=layout, seed=nheads)
+        w.context_lens = torch.tensor([900, 1, 257, 0, 640], dtype=torch.int32)
+        w.sinks = torch.linspace(-2, 2, nheads).to(w.query.dtype)
+        live = w.context_lens > 0
+        for kernel in ("fp8_loop", "fp8_reduce"):
+            for schedule in (0, 1):
+                bufs, _ = _run(w, kernel, schedule=schedule)
+                assert (bufs.out.cpu()[~live] == 0).all()
+                _check(bufs.out, w, oracle, f"{w.name}/{layout}/{kernel}/schedule{schedule}")
+                if kernel == "fp8_reduce" and schedule == 1:
+                    es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=w.partition_size,
+                                              max_num_partitions=w.max_num_partitions)
+                    for s in range(w.num_seqs):
+                        n = math.ceil(int(w.context_lens[s]) / w.partition_size)
+                        torch.testing.assert_close(bufs.max_logits[s, :, :n].cpu(), ml[s, :, :n], atol=1e-4, rtol=1e-5)
+                        torch.testing.assert_close(bufs.exp_sums[s, :, :n].cpu(), es[s, :, :n], atol=1e-4, rtol=1e-4)
+                        torch.testing.assert_close(bufs.tmp_out[s, :, :n].cpu(), tmp[s, :, :n], atol=2e-3, rtol=1e-2)
+                        assert torch.isnan(bufs.tmp_out[s, :, n:]).all()
