@@ -85,6 +85,19 @@ struct Pipeline {
   static constexpr bool stream_loads_split = (kKV8 ? FA_STREAM_LOADS_FP8_SPLIT : FA_STREAM_LOADS) != 0;
 };
 
+// Loop kernel that holds two column tiles per wavefront (paged_attention_loop_two_tile_kernel.h):
+// one work-group per compute unit, so each wavefront has to keep more bytes in flight by itself.
+#ifndef FA_TWO_TILE_TPC
+#define FA_TWO_TILE_TPC 2
+#endif
+#ifndef FA_TWO_TILE_TPC_FP8
+#define FA_TWO_TILE_TPC_FP8 FA_TPC_FP8
+#endif
+template <bool kKV8>
+struct TwoTile {
+  static constexpr int tiles_per_chunk = kKV8 ? FA_TWO_TILE_TPC_FP8 : FA_TWO_TILE_TPC;
+};
+
 // ---- persistent kernels (batches of up to 128 / 256 sequences) -------------------------
 // Split path, segment form: multi-wavefront work-groups take segments of several partitions
 // and write one partial per segment (paged_attention_segment_kernel.h).

@@ -151,6 +151,9 @@ struct WaveAttn {
   // EXT only: what column i stands for, and the position of its query token
   int col_q = 0, col_g = 0, col_last = 0;
   bool col_valid = false;
+  // EXT only, the same in every lane: the keys vis_lo .. vis_hi of the item at hand are seen by
+  // every query token of the launch (causal rule and local window)
+  int vis_lo = 0, vis_hi = -1;
 
   // Q^T as the MFMA "B" operand, one dword quad per k-step.  k-slot (r, e) of step c
   // stands for head-dim element qd(c, r) + e; K uses the same map.
@@ -217,6 +220,8 @@ struct WaveAttn {
     slope_log2 = x.slope_log2;
     out_mul = x.out_mul;
     col_last = ctx - p.query_len + col_q;
+    vis_hi = ctx - p.query_len + p.query_first;  // the launch's earliest query token
+    vis_lo = (p.mask_flags & kMaskWindow) ? vis_hi + p.query_count - 1 - p.window_left : 0;
   }
 
   // First chunk that holds a key some query token of the item sees (local window), at least c_begin.
@@ -421,8 +426,9 @@ struct WaveAttn {
                                         const TileScales *ts = nullptr) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
     float t[NT];
-    if (MASKS && p.mask_flags == 0 && p.query_len <= 1) {
-      // only scales asked for the extended instance: plain scores with the tiles' own scale
+    if (MASKS && !(p.mask_flags & (kMaskSoftcap | kMaskAlibi)) && ci * CT >= vis_lo && ci * CT + CT - 1 <= vis_hi) {
+      // no score modifier, and every query token of the launch sees the whole chunk (all but the
+      // last chunks of an item): plain scores with the tiles' own scale
       float k2[TPC];
 #pragma unroll
       for (int tl = 0; tl < TPC; ++tl) k2[tl] = ts->k[tl] * kLog2e;
@@ -433,14 +439,18 @@ struct WaveAttn {
       const float inv_cap2 = 2.0f * kLog2e / p.softcap;  // exp(2x/cap) = exp2(x * inv_cap2)
       const int first_visible = (p.mask_flags & kMaskWindow) ? col_last - p.window_left : 0;
 #pragma unroll
-      for (int e = 0; e < NT; ++e) {
-        float x = s.v[e >> 2][e & 3] * ts->k[e >> 2];
-        if (cap) {  // cap * tanh(x / cap), tanh(z) = 1 - 2 / (exp(2z) + 1)
-          const float e2 = fast_exp2(x * inv_cap2);
-          x = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f));
+      for (int e = 0; e < NT; ++e) t[e] = s.v[e >> 2][e & 3] * ts->k[e >> 2];
+      if (cap) {  // cap * tanh(x / cap), tanh(z) = 1 - 2 / (exp(2z) + 1); a loop of its own: stays a branch
+#pragma unroll
+        for (int e = 0; e < NT; ++e) {
+          const float e2 = fast_exp2(t[e] * inv_cap2);
+          t[e] = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f));
         }
+      }
+#pragma unroll
+      for (int e = 0; e < NT; ++e) {
         const int tok = ci * CT + (e >> 2) * kTileTokens + 4 * r + (e & 3);
-        x = x * kLog2e + slope_log2 * (float)(tok - col_last);
+        const float x = t[e] * kLog2e + slope_log2 * (float)(tok - col_last);
         t[e] = (tok < first_visible || tok > col_last) ? -INFINITY : x;
       }
     } else {
