@@ -35,6 +35,7 @@ __device__ __forceinline__ void merge_and_store(W &wa, const PagedAttnParams &p,
   constexpr int SL = NR / NW;
   static_assert(NR % NW == 0 && SL >= 2, "output slice per wavefront must hold >= 2 elements");
   const int r = wa.r, i = wa.i;
+  wa.settle();
   wa.l = rows_sum(wa.l);
   float M = wa.m, L = wa.l;
   float o[SL];

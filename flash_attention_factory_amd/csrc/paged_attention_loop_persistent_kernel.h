@@ -148,6 +148,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   // A wavefront's state of item n goes to LDS and the wavefront moves on; nobody waits here.
   auto publish = [&](int item) {
     const int b = item & 1;
+    wa.settle();
     wa.l = rows_sum(wa.l);
     if (r == 0) {
       sm_m[tile][b][wave][i] = wa.m;

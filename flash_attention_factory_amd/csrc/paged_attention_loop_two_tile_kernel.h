@@ -7,11 +7,27 @@
 // and V is loaded once, every operand is built once and feeds the MFMAs of both tiles
 // (WaveAttn::qk_two, pv_two), each tile keeps its own queries, softmax state and accumulators,
 // masks by its own columns' positions and is merged and stored for itself.  K and V cross HBM
-// and the caches exactly once per launch, and all four wavefronts of a work-group interleave an
-// item's chunks as in the one-tile kernel.  The price is registers (two sets of queries and
-// accumulators: one work-group per compute unit) and twice the merge buffers in LDS.
+// and the caches exactly once per launch.  The price is registers (two sets of queries and
+// accumulators): one wavefront per SIMD, so nothing else hides a wavefront's waits for memory.
 //
-// Item order, deferred merge, prefetch across items: as in the one-tile kernel.
+// That is why a wavefront keeps TWO chunks in registers (R0, R1: chunk j of an item sits in
+// R(j & 1)): while chunk j is computed, chunk j+1 is on its way, and as soon as the scores (the
+// values) of chunk j are out, K (V) of chunk j+2 is requested into the registers just freed.
+// Every load has a chunk and a half of compute to arrive.  Across items: the first chunk of the
+// next item is requested into R0 by the last step of the current item that uses R0, together
+// with what the item needs beyond K and V (queries, sinks, per-item multipliers).
+//
+// The wait counts in front of the MFMAs are fixed when the kernel is compiled, for the worst of
+// all paths that lead there; a path on which a load was skipped is one on which the registers
+// about to be used hold the newest load, and the count would be zero.  So the loop that runs
+// for most of an item (`steady`) requests its loads unconditionally, is entered only from code
+// that has requested both register sets, and contains neither stores nor LDS traffic; the one to
+// three chunks that end an item (or make up a short one) go through steps with conditions.
+//
+// Item order (longest first, dealt in a snake over the work-groups) and the merge through LDS
+// without barriers (publish / finish, one arrival counter per buffer): as in the one-tile kernel,
+// except that the merge owed to item n-1 is done at the end of item n, just before its own
+// states are published, so that no store and no wait for other wavefronts sits in the stream.
 #pragma once
 
 #include "paged_attention_loop_persistent_kernel.h"
@@ -84,9 +100,11 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       rank1 += ku > key1;
     }
   }
-  struct Item { int seq, kvh, ctx, c_end, c_lo; };  // c_lo: first chunk to read (0 unless EXT)
+  W wa(p, lane, 0), wb(p, lane, 1);  // the two column tiles
+  const int r = wa.r, i = wa.i;
+  struct Item { int seq, kvh, ctx, c_end, c_lo; };  // c_lo: first chunk some query token sees (local window)
   // n-th item of this work-group: position n*G + j on even n, n*G + G-1-j on odd n
-  auto item_at = [&](int n, Item &it) -> bool {
+  auto item_at = [&](int n, Item &it) __attribute__((always_inline)) -> bool {
     const int pos = n * G + ((n & 1) ? G - 1 - wg : wg);
     if (pos >= T) return false;
     const int rho = __builtin_amdgcn_readfirstlane(pos / Hk);
@@ -97,7 +115,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     it.seq = __builtin_amdgcn_readfirstlane(s);
     it.ctx = s < 64 ? __builtin_amdgcn_readlane(len0, s) : __builtin_amdgcn_readlane(len1, s - 64);
     it.c_end = (it.ctx + CT - 1) / CT;
-    it.c_lo = 0;
+    it.c_lo = wa.first_visible_chunk(it.ctx, 0);  // the launch's earliest query token decides: the same for both tiles
     return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
   };
 
@@ -107,19 +125,14 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   __shared__ float sm_acc[2][2][NW][NR][64];
   __shared__ int sm_arrived[2];  // wavefronts that have published (both tiles) into the buffer, ever
 
-  W wa(p, lane, 0), wb(p, lane, 1);  // the two column tiles
-  const int r = wa.r, i = wa.i;
-  Chunk R;
-
-  int n = 0;
-  Item cur;
-  if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
-  cur.c_lo = wa.first_visible_chunk(cur.ctx, 0);  // the launch's earliest query token decides: the same for both tiles
+  Item first;
+  if (!item_at(0, first)) return;  // the same for every wavefront of the work-group
   if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
   // A wavefront's states of item n go to LDS and the wavefront moves on; nobody waits here.
-  auto publish_tile = [&](W &w, int tile, int b) {
+  auto publish_tile = [&](W &w, int tile, int b) __attribute__((always_inline)) {
+    w.settle();
     w.l = rows_sum(w.l);
     if (r == 0) {
       sm_m[tile][b][wave][i] = w.m;
@@ -128,7 +141,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
 #pragma unroll
     for (int k = 0; k < NR; ++k) sm_acc[tile][b][wave][k][lane] = w.acc_at(k);
   };
-  auto publish = [&](int item) {
+  auto publish = [&](int item) __attribute__((always_inline)) {
     const int b = item & 1;
     publish_tile(wa, 0, b);
     publish_tile(wb, 1, b);
@@ -136,7 +149,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     if (lane == 0) __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
-  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, float out_mul) {
+  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, float out_mul) __attribute__((always_inline)) {
     float M = -INFINITY;
 #pragma unroll
     for (int v = 0; v < NW; ++v) M = fmaxf(M, sm_m[tile][b][v][i]);
@@ -164,9 +177,12 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
     }
   };
-  // Called one chunk into the following item (or after the last item): see the one-tile kernel for
-  // why the wait always ends and why a buffer is never overwritten while somebody still reads it.
-  auto finish = [&](int item, int seq, int kvh, float out_mul) {
+  // Every wavefront runs  ... finish(n-2), publish(n-1), finish(n-1), publish(n) ...  in this order.
+  // finish(n-1) waits for the publish(n-1) of all wavefronts, none of which waits for anything
+  // later than finish(n-2): the wait ends.  And publish(n) overwrites the buffer of item n-2 only
+  // after finish(n-1) has seen every wavefront's publish(n-1), which each of them issues after
+  // its finish(n-2).
+  auto finish = [&](int item, int seq, int kvh, float out_mul) __attribute__((always_inline)) {
     const int b = item & 1;
     const int target = NW * ((item >> 1) + 1);
     bool arrived = false;
@@ -183,21 +199,20 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     finish_tile(wa, 0, b, seq, kvh, out_mul);
     finish_tile(wb, 1, b, seq, kvh, out_mul);
   };
-  // one chunk of the current item through both tiles
-  auto scores_of = [&](Scores &sa, Scores &sb) { W::qk_two(wa, wb, R, sa, sb); };
-  auto soft_pv = [&](auto tail, const Scores &sa, const Scores &sb, int ci, int ctx, const TileScales &ts) {
-    const auto pa = wa.template soft<decltype(tail)::value, true>(R, sa, ci, ctx, &ts);
-    const auto pb = wb.template soft<decltype(tail)::value, true>(R, sb, ci, ctx, &ts);
-    W::pv_two(wa, wb, R, pa, pb);
-  };
-  auto table_of = [&](int seq) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
+  auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
+  // this wavefront's chunks of an item: c_lo + wave, + NW, ... below c_end
+  auto count_of = [&](const Item &it) __attribute__((always_inline)) { return max(0, (it.c_end - it.c_lo - wave + NW - 1) / NW); };
 
-  // first chunk of the first item
-  bool armed = cur.c_lo + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  Chunk R0, R1;
+  TileScales ts0 = {}, ts1 = {};  // multipliers of the chunks in R0, R1
+
+  int n = 0;
+  Item cur = first;
+  int m = count_of(cur);  // chunks of `cur` this wavefront computes; the first is in flight in R0 if there is one
   ItemExt cur_a = wa.fetch_item_ext(cur.kvh, table_of(cur.seq)), cur_b = wb.fetch_item_ext(cur.kvh, table_of(cur.seq));
   ItemExt nxt_a = {}, nxt_b = {};
-  TileScales ts = {}, nts = {}, nxt_ts = {};
-  if (armed) {
+  Ids ids1 = {};  // block ids of the item's second chunk, requested an item early
+  if (m > 0) {
     Ids ids;
 #pragma unroll
     for (int t = 0; t < TPC; ++t) {
@@ -207,11 +222,12 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     }
     if (cur.c_lo != 0)  // the ids requested with the lengths are those of chunk `wave`
       ids = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave, col_max);
+    ids1 = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave + NW, col_max);
     wa.load_q(cur.seq, cur.kvh);
     wb.load_q(cur.seq, cur.kvh);
-    wa.issue_k(R, cur.kvh, cur.c_lo + wave, ids);
-    wa.issue_v(R, cur.kvh, cur.c_lo + wave, ids);
-    ts = wa.fetch_scales(ids, cur.kvh, cur_a);
+    wa.issue_k(R0, cur.kvh, cur.c_lo + wave, ids);
+    wa.issue_v(R0, cur.kvh, cur.c_lo + wave, ids);
+    ts0 = wa.fetch_scales(ids, cur.kvh, cur_a);
   }
   uint32_t sink_a = wa.load_sink(cur.kvh, wave == 0), sink_b = wb.load_sink(cur.kvh, wave == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
@@ -220,15 +236,18 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   while (true) {
     Item nxt;
     const bool has_next = item_at(n + 1, nxt);
+    int next_m = 0;
     if (has_next) {
-      nxt.c_lo = wa.first_visible_chunk(nxt.ctx, 0);
+      next_m = count_of(nxt);
       nxt_a = wa.fetch_item_ext(nxt.kvh, table_of(nxt.seq));
       nxt_b = wb.fetch_item_ext(nxt.kvh, table_of(nxt.seq));
     }
-    const bool next_armed = has_next && nxt.c_lo + wave < nxt.c_end;
-    Ids nxt_ids = {};
-    if (next_armed) nxt_ids = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + wave, col_max);
-
+    const bool next_armed = next_m > 0;
+    Ids nxt_ids = {}, nxt_ids1 = {};
+    if (next_armed) {
+      nxt_ids = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + wave, col_max);
+      nxt_ids1 = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + wave + NW, col_max);
+    }
     wa.reset(sink_a);
     wb.reset(sink_b);
     wa.set_item(cur_a, cur.ctx);
@@ -238,63 +257,123 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       next_a = wa.load_sink(nxt.kvh, wave == 0);
       next_b = wb.load_sink(nxt.kvh, wave == 0);
     }
-    bool owed = n > 0;
-    if (armed) {
-      const int32_t *table = table_of(cur.seq);
-      int ci = cur.c_lo + wave;
-      Ids nids = wa.fetch_ids(table, ci + NW, col_max);
-      Scores sa, sb;
-      bool first = true;
-      while (ci + NW < cur.c_end) {  // the next chunk belongs to the same item
-        const int cn = ci + NW;
-        scores_of(sa, sb);
-        wa.issue_k(R, cur.kvh, cn, nids);
-        nts = wa.fetch_scales(nids, cur.kvh, cur_a);
-        soft_pv(std::false_type{}, sa, sb, ci, cur.ctx, ts);
-        wa.issue_v(R, cur.kvh, cn, nids);
-        nids = wa.fetch_ids(table, cn + NW, col_max);
-        ts = nts;
-        ci = cn;
-        if (first && owed) {  // one chunk into the item: the merge owed to the previous item
-          finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
-          owed = false;
-        }
-        first = false;
-      }
-      // last chunk of this wavefront in `cur`: what goes out next belongs to `nxt`
-      scores_of(sa, sb);
-      if (next_armed) {
-        wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
-        wb.load_q(nxt.seq, nxt.kvh);
-        next_a = wa.load_sink(nxt.kvh, wave == 0);
-        next_b = wb.load_sink(nxt.kvh, wave == 0);
-        wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-        nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
-      }
-      soft_pv(std::true_type{}, sa, sb, ci, cur.ctx, ts);
-      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-    } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
+    // What the next item needs beyond K and V, once the last scores of this one are out.
+    auto request_next_item = [&]() __attribute__((always_inline)) {
       wa.load_q(nxt.seq, nxt.kvh);
       wb.load_q(nxt.seq, nxt.kvh);
       next_a = wa.load_sink(nxt.kvh, wave == 0);
       next_b = wb.load_sink(nxt.kvh, wave == 0);
-      wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-      wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-      nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
+    };
+    TileScales nts = {};
+    if (m > 0) {
+      const int32_t *table = table_of(cur.seq);
+      const int c0 = cur.c_lo + wave;  // chunk j of the wavefront is chunk c0 + j * NW of the item
+      Scores sa, sb;
+      Ids ids_a = {}, ids_b = {};  // ids of the chunks R0 and R1 take next
+      int j = 0;
+      if (m >= 4) {
+        wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
+        wa.issue_v(R1, cur.kvh, c0 + NW, ids1);
+        ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
+        ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
+        ids_b = wa.fetch_ids(table, c0 + 3 * NW, col_max);
+        // steady: chunk j in R0 and j+1 in R1 are computed, chunks j+2 and j+3 requested
+        while (j + 3 < m) {
+          const int ca = c0 + j * NW, cb = ca + NW;
+          W::qk_two(wa, wb, R0, sa, sb);
+          wa.issue_k(R0, cur.kvh, ca + 2 * NW, ids_a);
+          nts = wa.fetch_scales(ids_a, cur.kvh, cur_a);
+          {
+            const auto pa = wa.template soft<false, true>(R0, sa, ca, cur.ctx, &ts0);
+            const auto pb = wb.template soft<false, true>(R0, sb, ca, cur.ctx, &ts0);
+            W::pv_two(wa, wb, R0, pa, pb);
+          }
+          wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
+          ts0 = nts;
+          ids_a = wa.fetch_ids(table, ca + 4 * NW, col_max);
+
+          W::qk_two(wa, wb, R1, sa, sb);
+          wa.issue_k(R1, cur.kvh, cb + 2 * NW, ids_b);
+          nts = wa.fetch_scales(ids_b, cur.kvh, cur_a);
+          {
+            const auto pa = wa.template soft<false, true>(R1, sa, cb, cur.ctx, &ts1);
+            const auto pb = wb.template soft<false, true>(R1, sb, cb, cur.ctx, &ts1);
+            W::pv_two(wa, wb, R1, pa, pb);
+          }
+          wa.issue_v(R1, cur.kvh, cb + 2 * NW, ids_b);
+          ts1 = nts;
+          ids_b = wa.fetch_ids(table, cb + 4 * NW, col_max);
+          j += 2;
+        }
+      } else if (m >= 2) {
+        wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
+        wa.issue_v(R1, cur.kvh, c0 + NW, ids1);
+        ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
+        if (m == 3) ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
+      }
+      // The one to three chunks that end the item: j in R0, j+1 in R1, j+2 on its way into R0 or
+      // requested now.  The last of these steps that uses R0 requests the next item's first chunk.
+      const int rem = m - j;
+      const int ca = c0 + j * NW;
+      {
+        W::qk_two(wa, wb, R0, sa, sb);
+        if (rem == 3) {
+          wa.issue_k(R0, cur.kvh, ca + 2 * NW, ids_a);
+          nts = wa.fetch_scales(ids_a, cur.kvh, cur_a);
+        } else if (next_armed) {
+          if (rem == 1) request_next_item();
+          wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+          nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
+        }
+        const auto pa = wa.template soft<true, true>(R0, sa, ca, cur.ctx, &ts0);
+        const auto pb = wb.template soft<true, true>(R0, sb, ca, cur.ctx, &ts0);
+        W::pv_two(wa, wb, R0, pa, pb);
+        if (rem == 3) {
+          wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
+        } else if (next_armed) {
+          wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+        }
+        ts0 = nts;
+      }
+      if (rem >= 2) {
+        W::qk_two(wa, wb, R1, sa, sb);
+        if (rem == 2 && next_armed) request_next_item();
+        const auto pa = wa.template soft<true, true>(R1, sa, ca + NW, cur.ctx, &ts1);
+        const auto pb = wb.template soft<true, true>(R1, sb, ca + NW, cur.ctx, &ts1);
+        W::pv_two(wa, wb, R1, pa, pb);
+      }
+      if (rem == 3) {
+        W::qk_two(wa, wb, R0, sa, sb);
+        if (next_armed) {
+          request_next_item();
+          wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+          nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
+        }
+        const auto pa = wa.template soft<true, true>(R0, sa, ca + 2 * NW, cur.ctx, &ts0);
+        const auto pb = wb.template soft<true, true>(R0, sb, ca + 2 * NW, cur.ctx, &ts0);
+        W::pv_two(wa, wb, R0, pa, pb);
+        if (next_armed) wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+        ts0 = nts;
+      }
+    } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
+      request_next_item();
+      wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      ts0 = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
     }
-    if (owed) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
+    if (n > 0) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
     publish(n);
 
     if (!has_next) break;
     prev = cur;
+    prev_out_mul = cur_a.out_mul;
     cur = nxt;
-    armed = next_armed;
+    m = next_m;
+    ids1 = nxt_ids1;
     sink_a = next_a;
     sink_b = next_b;
-    prev_out_mul = cur_a.out_mul;
     cur_a = nxt_a;
     cur_b = nxt_b;
-    ts = nxt_ts;
     ++n;
   }
   finish(n, cur.seq, cur.kvh, cur_a.out_mul);

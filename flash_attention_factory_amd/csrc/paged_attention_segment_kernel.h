@@ -175,6 +175,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
 
   auto publish = [&](int n) {
     const int b = n & 1;
+    wa.settle();
     wa.l = rows_sum(wa.l);
     if (r == 0) {
       sm_m[tile][b][wave][i] = wa.m;

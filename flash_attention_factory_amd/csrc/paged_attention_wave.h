@@ -158,10 +158,17 @@ struct WaveAttn {
   // Q^T as the MFMA "B" operand, one dword quad per k-step.  k-slot (r, e) of step c
   // stands for head-dim element qd(c, r) + e; K uses the same map.
   u32x4 qB[KSTEPS];
-  // Online softmax state.  m: running max (base-2 units) of head i, identical in the four
-  // rows r.  l: this lane's share of the running sum (its own tokens).
+  // Online softmax state.  mt: running max (base-2 units) of head i, identical in the four
+  // rows r.  m: the reference the sums are taken against, exp2(score - m); it follows mt only
+  // when it has fallen behind by more than kRescaleSlack, because every change of m costs a
+  // pass over the accumulators (with a handful of heads or query tokens in the 16 columns some
+  // column sets a new maximum in nearly every chunk, by a small step).  Until then the
+  // probabilities may exceed 1, by a factor of at most 2^kRescaleSlack: well inside the range
+  // of fp16 and bf16, and sums and accumulators are fp32.  settle() brings m up to mt.
+  // l: this lane's share of the running sum (its own tokens).
   // acc[dt][e]: O^T[d = (4r+e)*NDT + dt][head i], un-normalised.
-  float m, l;
+  static constexpr float kRescaleSlack = 8.0f;
+  float m, mt, l;
   f32x4 acc[NDT];
   float slope_log2 = 0.f;  // ALiBi slope of head i in base-2 units (MASKS instances only)
   // EXT: what the normalised output of the item at hand is multiplied with (see ItemExt).
@@ -293,8 +300,22 @@ struct WaveAttn {
       m = load_scalar16<QT>(&h) * kLog2e;
       l = (r == 0) ? 1.f : 0.f;
     }
+    mt = m;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Sums and accumulators relative to the true maximum: the state every merge, publish and store
+  // starts from (m is what max_logits and the merges see).
+  __device__ __forceinline__ void settle() {
+    if (__any(mt != m)) {
+      const float m_sub = (mt == -INFINITY) ? 0.f : mt;
+      const float alpha = fast_exp2(m - m_sub);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+      m = mt;
+    }
   }
 
   // Physical block id of every 16-token tile of chunk ci of a sequence's table row.
@@ -475,23 +496,29 @@ struct WaveAttn {
 #pragma unroll
     for (int e = 1; e < NT; ++e) mx = fmaxf(mx, t[e]);
     mx = rows_max(mx);
-    const float m_new = fmaxf(m, mx);
-    // MASKS: a column may see nothing of a chunk (a query token before the chunk's keys)
-    // and nothing before it either; subtract 0 then, so that -inf stays -inf, not NaN
-    const float m_sub = (MASKS && m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m - m_sub);  // exp2(-inf) = 0 on the first chunk
+    mt = fmaxf(mt, mx);
+    // the reference follows when some column's has fallen too far behind (on the first chunk: has
+    // none yet, inf > slack; a column that has seen nothing so far: -inf - -inf = NaN, no)
+    // (per-block V scales ride on the probabilities and may be large: no slack to spare there)
+    const float slack = (MASKS && KV8 && p.kv_scale_mode == kScaleBlock) ? 0.f : kRescaleSlack;
+    if (__any(mt - m > slack)) {
+      // MASKS: a column may see nothing of a chunk (a query token before the chunk's keys)
+      // and nothing before it either; subtract 0 then, so that -inf stays -inf, not NaN
+      const float m_to = (MASKS && mt == -INFINITY) ? 0.f : mt;
+      const float alpha = fast_exp2(m - m_to);  // exp2(-inf) = 0 on the first chunk
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+      m = mt;
+    }
+    const float m_sub = (MASKS && m == -INFINITY) ? 0.f : m;
     float ps = 0.f;
 #pragma unroll
     for (int e = 0; e < NT; ++e) {
       t[e] = fast_exp2(t[e] - m_sub);
       ps += t[e];
     }
-    l = l * alpha + ps;
-    m = m_new;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
-    }
+    l += ps;
     // k-slots (r, e) of step pr = this lane's eight tokens of the step, rounded to the q
     // dtype (paged_attention_kernel_loop.hpp:404-407)
     if constexpr (MASKS && KV8) {  // per-block V scales ride on the probabilities (1.0 otherwise)

@@ -143,11 +143,16 @@ def test_schedule_option(oracle, fp8, schedule):
         if "reduce" in kernel:
             es, ml, tmp = call_oracle(oracle.kernel_partition, w, partition_size=w.partition_size,
                                       max_num_partitions=w.max_num_partitions)
+            # The kernels round the probabilities to the query dtype against a reference maximum that
+            # may lag the true one by a few units, the oracle against the true one: the same values,
+            # rounded differently.  bf16 keeps 8 significant bits, and a partition of one or a few
+            # tokens does not average that out.
+            tmp_atol = 2e-3 if w.query.dtype == torch.float16 else 4e-3
             for s in range(w.num_seqs):
                 live = math.ceil(int(w.context_lens[s]) / w.partition_size)
                 torch.testing.assert_close(bufs.max_logits[s, :, :live].cpu(), ml[s, :, :live], atol=1e-4, rtol=1e-5)
                 torch.testing.assert_close(bufs.exp_sums[s, :, :live].cpu(), es[s, :, :live], atol=1e-4, rtol=1e-4)
-                torch.testing.assert_close(bufs.tmp_out[s, :, :live].cpu(), tmp[s, :, :live], atol=2e-3, rtol=1e-2)
+                torch.testing.assert_close(bufs.tmp_out[s, :, :live].cpu(), tmp[s, :, :live], atol=tmp_atol, rtol=1e-2)
                 assert torch.isnan(bufs.max_logits[s, :, live:]).all()
 
 
