@@ -205,6 +205,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
 
   Chunk R0, R1;
   TileScales ts0 = {}, ts1 = {};  // multipliers of the chunks in R0, R1
+  bool k1_ready = false;          // K of the item's second chunk has been requested into R1 already
+  constexpr int kWaitVmcnt0 = 0x0F70;  // s_waitcnt vmcnt(0), no wait on the other counters
 
   int n = 0;
   Item cur = first;
@@ -272,47 +274,80 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       Ids ids_a = {}, ids_b = {};  // ids of the chunks R0 and R1 take next
       int j = 0;
       if (m >= 4) {
-        wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
-        wa.issue_v(R1, cur.kvh, c0 + NW, ids1);
+        // The second chunk: K now; its V loads go out between the MFMAs of the first chunk's scores.
+        int64_t vp0[TPC], vp1[TPC];  // where the V loads that R0 / R1 still wait for read from
+        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
+#pragma unroll
+        for (int t = 0; t < TPC; ++t) vp1[t] = wa.v_tile_at(cur.kvh, c0 + NW, t, ids1);
         ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
         ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
         ids_b = wa.fetch_ids(table, c0 + 3 * NW, col_max);
+        // One chunk: X holds chunk cx; the chunk two further on takes X over.  A wavefront that has
+        // to wait at a load (the memory pipeline is full most of the time) computes nothing
+        // meanwhile and there is no second wavefront on its SIMD, so the loads go out one at a
+        // time between pieces of arithmetic: the V loads the OTHER set still waits for between
+        // the MFMAs of the scores, the K loads of X's next chunk along softmax and P.V.
+        auto steady = [&](Chunk &X, TileScales &tsx, int64_t (&vpx)[TPC], Chunk &Y, const int64_t (&vpy)[TPC], int cx,
+                          Ids &ids) __attribute__((always_inline)) {
+          constexpr int NS = W::KSTEPS * TPC, NV = 4 * TPC, NK = W::KL * TPC;
+          W::qk_two(wa, wb, X, sa, sb, [&](int slot) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = slot * NV / NS; v < (slot + 1) * NV / NS; ++v) {
+              __builtin_amdgcn_sched_barrier(0);
+              wa.load_v_one(Y, v / 4, v % 4, vpy[v / 4]);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          });
+          int64_t kp[TPC];
+#pragma unroll
+          for (int t = 0; t < TPC; ++t) {
+            kp[t] = wa.k_tile_at(cur.kvh, cx + 2 * NW, t, ids);
+            vpx[t] = wa.v_tile_at(cur.kvh, cx + 2 * NW, t, ids);
+          }
+          nts = wa.fetch_scales(ids, cur.kvh, cur_a);
+          ids = wa.fetch_ids(table, cx + 4 * NW, col_max);
+          auto k_loads = [&](int part) __attribute__((always_inline)) {  // quarter `part` of the NK loads
+#pragma unroll
+            for (int k = part * NK / 4; k < (part + 1) * NK / 4; ++k) {
+              __builtin_amdgcn_sched_barrier(0);
+              wa.load_k_one(X, k / W::KL, k % W::KL, kp[k / W::KL]);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          };
+          k_loads(0);
+          const auto pa = wa.template soft<false, true>(X, sa, cx, cur.ctx, &tsx);
+          k_loads(1);
+          const auto pb = wb.template soft<false, true>(X, sb, cx, cur.ctx, &tsx);
+          k_loads(2);
+          W::pv_two(wa, wb, X, pa, pb, [&](int slot) __attribute__((always_inline)) {
+            if (slot == W::NP2 * W::NDT / 2 - 1) k_loads(3);
+          });
+          tsx = nts;
+        };
+        // Everything requested so far has to arrive before the loop is entered: most of it was
+        // requested a step or more ago, and what the loop then waits for is decided by its own
+        // loads alone, not by the worst of the paths that lead here (on some of which the
+        // requests above were skipped).
+        __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
         // steady: chunk j in R0 and j+1 in R1 are computed, chunks j+2 and j+3 requested
         while (j + 3 < m) {
-          const int ca = c0 + j * NW, cb = ca + NW;
-          W::qk_two(wa, wb, R0, sa, sb);
-          wa.issue_k(R0, cur.kvh, ca + 2 * NW, ids_a);
-          nts = wa.fetch_scales(ids_a, cur.kvh, cur_a);
-          {
-            const auto pa = wa.template soft<false, true>(R0, sa, ca, cur.ctx, &ts0);
-            const auto pb = wb.template soft<false, true>(R0, sb, ca, cur.ctx, &ts0);
-            W::pv_two(wa, wb, R0, pa, pb);
-          }
-          wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
-          ts0 = nts;
-          ids_a = wa.fetch_ids(table, ca + 4 * NW, col_max);
-
-          W::qk_two(wa, wb, R1, sa, sb);
-          wa.issue_k(R1, cur.kvh, cb + 2 * NW, ids_b);
-          nts = wa.fetch_scales(ids_b, cur.kvh, cur_a);
-          {
-            const auto pa = wa.template soft<false, true>(R1, sa, cb, cur.ctx, &ts1);
-            const auto pb = wb.template soft<false, true>(R1, sb, cb, cur.ctx, &ts1);
-            W::pv_two(wa, wb, R1, pa, pb);
-          }
-          wa.issue_v(R1, cur.kvh, cb + 2 * NW, ids_b);
-          ts1 = nts;
-          ids_b = wa.fetch_ids(table, cb + 4 * NW, col_max);
+          steady(R0, ts0, vp0, R1, vp1, c0 + j * NW, ids_a);
+          steady(R1, ts1, vp1, R0, vp0, c0 + (j + 1) * NW, ids_b);
           j += 2;
         }
+        // the V loads R1 still waits for
+#pragma unroll
+        for (int v = 0; v < 4 * TPC; ++v) wa.load_v_one(R1, v / 4, v % 4, vp1[v / 4]);
       } else if (m >= 2) {
-        wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
+        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
         wa.issue_v(R1, cur.kvh, c0 + NW, ids1);
         ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
         if (m == 3) ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
       }
       // The one to three chunks that end the item: j in R0, j+1 in R1, j+2 on its way into R0 or
-      // requested now.  The last of these steps that uses R0 requests the next item's first chunk.
+      // requested now.  The last of these steps that uses R0 requests the next item's first chunk,
+      // the step that uses R1 the K half of its second.
+      k1_ready = false;
       const int rem = m - j;
       const int ca = c0 + j * NW;
       {
@@ -338,6 +373,10 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       if (rem >= 2) {
         W::qk_two(wa, wb, R1, sa, sb);
         if (rem == 2 && next_armed) request_next_item();
+        if (next_m >= 2) {
+          wa.issue_k(R1, nxt.kvh, nxt.c_lo + wave + NW, nxt_ids1);
+          k1_ready = true;
+        }
         const auto pa = wa.template soft<true, true>(R1, sa, ca + NW, cur.ctx, &ts1);
         const auto pb = wb.template soft<true, true>(R1, sb, ca + NW, cur.ctx, &ts1);
         W::pv_two(wa, wb, R1, pa, pb);
@@ -356,6 +395,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
         ts0 = nts;
       }
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
+      k1_ready = false;
       request_next_item();
       wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
       wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);

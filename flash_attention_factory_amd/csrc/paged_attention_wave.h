@@ -337,33 +337,48 @@ struct WaveAttn {
   }
 
   // K and V of a chunk go out separately so that either half of the register set can be
-  // refilled as soon as it has been consumed.
+  // refilled as soon as it has been consumed.  k_tile_at / v_tile_at: where this lane reads in
+  // tile t of the chunk, as a byte offset into the pool (an offset, not a pointer: a pointer kept
+  // across loop iterations loses its address space and the loads become flat loads);
+  // load_k_one / load_v_one: one load instruction from there (KL per tile for K, four token rows
+  // per tile for V), for kernels that spread a chunk's loads over the arithmetic of another.
+  __device__ __forceinline__ int64_t k_tile_at(int kvh, int ci, int t, const Ids &ids) const {
+    if constexpr (kRowLoads) {
+      // load c brings line c >> 1 of the rows 8 (c & 1) .. 8 (c & 1) + 7 whole: the lanes (r, i)
+      // and (r, i ^ 8) share a row
+      return tile_offset(kvh, ci, t, ids) + (int64_t)(i & 7) * p.kv_token_bytes + (i >> 3) * 64 + r * 16;
+    } else {
+      return tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
+    }
+  }
+  __device__ __forceinline__ void load_k_one(Chunk &R, int t, int c, int64_t at) const {
+    const char *kp = p.key_cache + at;
+    if constexpr (kRowLoads) {
+      R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + (int64_t)(8 * (c & 1)) * p.kv_token_bytes + (c >> 1) * 128));
+    } else {
+      R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + c * 64));
+    }
+  }
+  __device__ __forceinline__ int64_t v_tile_at(int kvh, int ci, int t, const Ids &ids) const {
+    return tile_offset(kvh, ci, t, ids) + (int64_t)(4 * r) * p.kv_token_bytes + i * VB;
+  }
+  __device__ __forceinline__ void load_v_one(Chunk &R, int t, int e, int64_t at) const {
+    VLoad<VW, kStream>::ld(R.v[t * 4 + e], p.value_cache + at + e * p.kv_token_bytes);
+  }
   __device__ __forceinline__ void issue_k(Chunk &R, int kvh, int ci, const Ids &ids) const {
 #pragma unroll
     for (int t = 0; t < TPC; ++t) {
-      if constexpr (kRowLoads) {
-        // load c brings line c >> 1 of the rows 8 (c & 1) .. 8 (c & 1) + 7 whole: the lanes (r, i)
-        // and (r, i ^ 8) share a row
-        const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)(i & 7) * p.kv_token_bytes +
-                         (i >> 3) * 64 + r * 16;
+      const int64_t at = k_tile_at(kvh, ci, t, ids);
 #pragma unroll
-        for (int c = 0; c < KL; ++c)
-          R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(
-              kp + (int64_t)(8 * (c & 1)) * p.kv_token_bytes + (c >> 1) * 128));
-      } else {
-        const char *kp = p.key_cache + tile_offset(kvh, ci, t, ids) + (int64_t)i * p.kv_token_bytes + r * 16;
-#pragma unroll
-        for (int c = 0; c < KL; ++c) R.k[t][c] = kv_load<kStream>(reinterpret_cast<const u32x4 *>(kp + c * 64));
-      }
+      for (int c = 0; c < KL; ++c) load_k_one(R, t, c, at);
     }
   }
   __device__ __forceinline__ void issue_v(Chunk &R, int kvh, int ci, const Ids &ids) const {
 #pragma unroll
     for (int t = 0; t < TPC; ++t) {
-      const char *vp = p.value_cache + tile_offset(kvh, ci, t, ids) +
-                       (int64_t)(4 * r) * p.kv_token_bytes + i * VB;
+      const int64_t at = v_tile_at(kvh, ci, t, ids);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) VLoad<VW, kStream>::ld(R.v[t * 4 + e], vp + e * p.kv_token_bytes);
+      for (int e = 0; e < 4; ++e) load_v_one(R, t, e, at);
     }
   }
 
@@ -501,7 +516,9 @@ struct WaveAttn {
     // none yet, inf > slack; a column that has seen nothing so far: -inf - -inf = NaN, no)
     // (per-block V scales ride on the probabilities and may be large: no slack to spare there)
     const float slack = (MASKS && KV8 && p.kv_scale_mode == kScaleBlock) ? 0.f : kRescaleSlack;
-    if (__any(mt - m > slack)) {
+    // (unlikely: where the accumulators live in AGPRs the copies to and from VGPRs that this
+    // block needs are then placed inside it, not in front of the branch)
+    if (__builtin_expect(__any(mt - m > slack), 0)) {
       // MASKS: a column may see nothing of a chunk (a query token before the chunk's keys)
       // and nothing before it either; subtract 0 then, so that -inf stays -inf, not NaN
       const float m_to = (MASKS && mt == -INFINITY) ? 0.f : mt;
@@ -545,7 +562,11 @@ struct WaveAttn {
 
   // Two column tiles held by ONE wavefront (a and b: the same chunk, different 16 columns) share
   // the K and V operands: every operand is built once and feeds both tiles' MFMAs.
-  static __device__ __forceinline__ void qk_two(const WaveAttn &a, const WaveAttn &b, Chunk &R, Scores &sa, Scores &sb) {
+  // `between(slot)` is called after the MFMAs of every (k-step, tile) pair, slot = c * TPC + t, and
+  // after those of every d-tile, slot = pr * NDT + dt: where a kernel places the loads of other chunks.
+  template <typename F>
+  static __device__ __forceinline__ void qk_two(const WaveAttn &a, const WaveAttn &b, Chunk &R, Scores &sa, Scores &sb,
+                                                F &&between) {
     if constexpr (kRowLoads) {
 #pragma unroll
       for (int t = 0; t < TPC; ++t)
@@ -561,9 +582,12 @@ struct WaveAttn {
         const u32x4 ko = a.k_operand(R, t, c);
         sa.v[t] = mfma_16x16x32<QT>(ko, a.qB[c], sa.v[t]);
         sb.v[t] = mfma_16x16x32<QT>(ko, b.qB[c], sb.v[t]);
+        between(c * TPC + t);
       }
   }
-  static __device__ __forceinline__ void pv_two(WaveAttn &a, WaveAttn &b, const Chunk &R, const Probs &pa, const Probs &pb) {
+  template <typename F>
+  static __device__ __forceinline__ void pv_two(WaveAttn &a, WaveAttn &b, const Chunk &R, const Probs &pa, const Probs &pb,
+                                                F &&between) {
 #pragma unroll
     for (int pr = 0; pr < NP2; ++pr)
 #pragma unroll
@@ -571,7 +595,14 @@ struct WaveAttn {
         const u32x4 vo = a.v_operand(R, pr, dt);
         a.acc[dt] = mfma_16x16x32<QT>(vo, pa.v[pr], a.acc[dt]);
         b.acc[dt] = mfma_16x16x32<QT>(vo, pb.v[pr], b.acc[dt]);
+        between(pr * NDT + dt);
       }
+  }
+  static __device__ __forceinline__ void qk_two(const WaveAttn &a, const WaveAttn &b, Chunk &R, Scores &sa, Scores &sb) {
+    qk_two(a, b, R, sa, sb, [](int) {});
+  }
+  static __device__ __forceinline__ void pv_two(WaveAttn &a, WaveAttn &b, const Chunk &R, const Probs &pa, const Probs &pb) {
+    pv_two(a, b, R, pa, pb, [](int) {});
   }
 
   // A lane's NR accumulator values are NR consecutive head-dim elements of head i:
