@@ -193,7 +193,8 @@ struct WaveAttn {
   // requests the values, so that a persistent kernel can ask for the next item's while the
   // current one still streams; set_item makes them the ones soft() works with.
   struct ItemExt {
-    float slope_log2;  // ALiBi slope of this lane's head, base-2 units
+    float slope;       // ALiBi slope of this lane's head as loaded (set_item converts it: arithmetic on
+                       // the value here would make the wavefront wait for the load where it is issued)
     float k_mul;       // raw score -> scaled score: softmax scale x K scale (tensor or head)
     float out_mul;     // what the normalised output is multiplied with: V scale (tensor or
                        // head), or with per-block scales the item's reference V scale
@@ -204,8 +205,8 @@ struct WaveAttn {
   // item's reference with per-block scales.
   __device__ __forceinline__ ItemExt fetch_item_ext(int kvh, const int32_t *table) const {
     ItemExt x;
-    x.slope_log2 =
-        ((p.mask_flags & kMaskAlibi) && col_valid) ? p.alibi_slopes[kvh * p.group + col_g] * kLog2e : 0.f;
+    x.slope = 0.f;
+    if ((p.mask_flags & kMaskAlibi) && col_valid) x.slope = p.alibi_slopes[kvh * p.group + col_g];
     x.k_mul = p.score_scale;
     x.out_mul = p.out_scale;
     x.inv_v_ref = 1.f;
@@ -224,7 +225,7 @@ struct WaveAttn {
 
   // Query token q of the item sits at position ctx - query_len + q and sees the keys up to there.
   __device__ __forceinline__ void set_item(const ItemExt &x, int ctx) {
-    slope_log2 = x.slope_log2;
+    slope_log2 = x.slope * kLog2e;
     out_mul = x.out_mul;
     col_last = ctx - p.query_len + col_q;
     vis_hi = ctx - p.query_len + p.query_first;  // the launch's earliest query token
@@ -521,11 +522,13 @@ struct WaveAttn {
     if (__builtin_expect(__any(mt - m > slack), 0)) {
       // MASKS: a column may see nothing of a chunk (a query token before the chunk's keys)
       // and nothing before it either; subtract 0 then, so that -inf stays -inf, not NaN
-      const float m_to = (MASKS && mt == -INFINITY) ? 0.f : mt;
-      const float alpha = fast_exp2(m - m_to);  // exp2(-inf) = 0 on the first chunk
-      l *= alpha;
+      if (__any(m != -INFINITY)) {  // on an item's first chunk (without sinks) sums and accumulators are still zero
+        const float m_to = (MASKS && mt == -INFINITY) ? 0.f : mt;
+        const float alpha = fast_exp2(m - m_to);  // exp2(-inf) = 0 for a column that has seen nothing so far
+        l *= alpha;
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+        for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+      }
       m = mt;
     }
     const float m_sub = (MASKS && m == -INFINITY) ? 0.f : m;
