@@ -21,13 +21,13 @@
 // all paths that lead there; a path on which a load was skipped is one on which the registers
 // about to be used hold the newest load, and the count would be zero.  So the loop that runs
 // for most of an item (`steady`) requests its loads unconditionally, is entered only from code
-// that has requested both register sets, and contains neither stores nor LDS traffic; the one to
-// three chunks that end an item (or make up a short one) go through steps with conditions.
+// that has requested both register sets; the one to three chunks that end an item (or make up a
+// short one) go through steps with conditions.
 //
 // Item order (longest first, dealt in a snake over the work-groups) and the merge through LDS
 // without barriers (publish / finish, one arrival counter per buffer): as in the one-tile kernel,
-// except that the merge owed to item n-1 is done at the end of item n, just before its own
-// states are published, so that no store and no wait for other wavefronts sits in the stream.
+// except that the merge owed to item n-1 is done one chunk into a long item n (its stores add
+// operations to one path into the loop's waits and cannot lower a count), else at its end.
 #pragma once
 
 #include "paged_attention_loop_persistent_kernel.h"
@@ -267,6 +267,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       next_b = wb.load_sink(nxt.kvh, wave == 0);
     };
     TileScales nts = {};
+    bool owed = n > 0;  // finish(n - 1) still to do
     if (m > 0) {
       const int32_t *table = table_of(cur.seq);
       const int c0 = cur.c_lo + wave;  // chunk j of the wavefront is chunk c0 + j * NW of the item
@@ -332,6 +333,10 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
         // steady: chunk j in R0 and j+1 in R1 are computed, chunks j+2 and j+3 requested
         while (j + 3 < m) {
           steady(R0, ts0, vp0, R1, vp1, c0 + j * NW, ids_a);
+          if (owed) {  // a chunk into the item, the next requests on their way: the merge owed to the item before
+            finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
+            owed = false;
+          }
           steady(R1, ts1, vp1, R0, vp0, c0 + (j + 1) * NW, ids_b);
           j += 2;
         }
@@ -401,7 +406,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
       ts0 = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
     }
-    if (n > 0) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
+    if (owed) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
     publish(n);
 
     if (!has_next) break;
