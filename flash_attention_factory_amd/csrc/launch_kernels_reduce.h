@@ -44,7 +44,7 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
                             shape.num_pool_blocks > 0 &&
                             (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
-  // columns, or in the segment form two tiles of 16 held by two halves of every work-group.
+  // columns, or in the segment form two tiles of 16 held by every wavefront.
   // Every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
   const int per_tile = p.query_count;
   const int per_launch = (segment_form && r.query_len > per_tile) ? 2 * per_tile : per_tile;
@@ -58,8 +58,8 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
                                              Pipeline<KV8>::tiles_per_chunk, false>;
       auto extended = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                                 Pipeline<KV8>::tiles_per_chunk, true>;
-      auto two_tiles = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                                 Pipeline<KV8>::tiles_per_chunk, true, 2>;
+      // two column tiles in the registers of every wavefront: K and V are loaded once for both
+      auto two_tiles = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, SW, TwoTile<KV8>::tiles_per_chunk, true, true>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
       if (q0 == 0) {
         // Every launch of the call gets the same number of work-groups: the segment length, which

@@ -30,15 +30,19 @@
 // operations to one path into the loop's waits and cannot lower a count), else at its end.
 #pragma once
 
+#include "paged_attention_items.h"
 #include "paged_attention_loop_persistent_kernel.h"
 
 namespace fa {
 
-template <int D, typename QT, int KVF, int NWG, int TPC, bool KROW = true>
+// PART: the split path.  Items are segments of partitions (SegmentItems), what is stored per item
+// and column is a partial -- max, sum and normalised values in exp_sums / max_logits / tmp_out at
+// the slot of the segment's first partition -- and the reduce kernel follows.
+template <int D, typename QT, int KVF, int NWG, int TPC, bool KROW = true, bool PART = false>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(1)))
 paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   constexpr int NW = NWG;  // wavefronts that share an item's chunks and merge
-  using W = WaveAttn<D, QT, KVF, TPC, Pipeline<(KVF != 0)>::stream_loads_loop, true, KROW>;
+  using W = WaveAttn<D, QT, KVF, TPC, PART ? SegmentSplit<(KVF != 0)>::stream_loads : Pipeline<(KVF != 0)>::stream_loads_loop, true, KROW>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   using ItemExt = typename W::ItemExt;
@@ -52,71 +56,22 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int S = p.num_seqs;
-  const int Hk = p.num_kv_heads;
-  const int T = S * Hk;
   const int G = gridDim.x;
   const int wg = blockIdx.x;
-  const int max_ctx = p.max_blocks_per_seq << p.block_shift;
   const int col_max = p.max_blocks_per_seq - 1;
 
-  // ---- rank the sequences by length, longest first; lane holds sequences lane, lane+64 --
-  // Requested together with the lengths, so that the first K/V loads depend on one round
-  // trip to memory, not two: for EVERY sequence, the block ids of the chunk this wavefront
-  // would start with.  Once the ranking has named the first item its ids are a lane away.
-  int len0 = -1, len1 = -1;
-  int sid0[TPC] = {}, sid1[TPC] = {};
-  if (lane < S) {
-    len0 = max(0, min(p.context_lens[lane], max_ctx));
-    const int32_t *row = p.block_tables + (int64_t)lane * p.max_blocks_per_seq;
-#pragma unroll
-    for (int t = 0; t < TPC; ++t) sid0[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
-  }
-  if (S > 64 && lane + 64 < S) {
-    len1 = max(0, min(p.context_lens[lane + 64], max_ctx));
-    const int32_t *row = p.block_tables + (int64_t)(lane + 64) * p.max_blocks_per_seq;
-#pragma unroll
-    for (int t = 0; t < TPC; ++t) sid1[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
-  }
-  // Sort key: length, then lower sequence number first; distinct for distinct sequences
-  // (lengths stay below 2^24, the launcher sees to that).  Lanes without a sequence: -1.
-  const int key0 = len0 < 0 ? -1 : (len0 << 7) | (127 - lane);
-  const int key1 = len1 < 0 ? -1 : (len1 << 7) | (63 - lane);
-  int rank0 = 0, rank1 = 0;  // how many sequences come before this one
-  // eight sequences per trip; lanes past the batch hold -1 and count for nothing
-  for (int u0 = 0; u0 < min(S, 64); u0 += 8) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int ku = __builtin_amdgcn_readlane(key0, u0 + j);
-      rank0 += ku > key0;
-      rank1 += ku > key1;
-    }
-  }
-  for (int u0 = 0; u0 < S - 64; u0 += 8) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int ku = __builtin_amdgcn_readlane(key1, u0 + j);
-      rank0 += ku > key0;
-      rank1 += ku > key1;
-    }
-  }
   W wa(p, lane, 0), wb(p, lane, 1);  // the two column tiles
   const int r = wa.r, i = wa.i;
-  struct Item { int seq, kvh, ctx, c_end, c_lo; };  // c_lo: first chunk some query token sees (local window)
-  // n-th item of this work-group: position n*G + j on even n, n*G + G-1-j on odd n
+  using Item = WorkItem;
+  std::conditional_t<PART, SegmentItems, LoopItems<TPC>> items;
+  if constexpr (PART) items.build(p, lane, G);
+  else items.build(p, lane, wave, G, CT);
+  // n-th item of this work-group, read from its first chunk that some query token of the launch
+  // sees (local window; the launch's earliest query token decides: the same for both tiles)
   auto item_at = [&](int n, Item &it) __attribute__((always_inline)) -> bool {
-    const int pos = n * G + ((n & 1) ? G - 1 - wg : wg);
-    if (pos >= T) return false;
-    const int rho = __builtin_amdgcn_readfirstlane(pos / Hk);
-    it.kvh = pos - rho * Hk;
-    const unsigned long long b0 = __ballot(key0 >= 0 && rank0 == rho);
-    const unsigned long long b1 = __ballot(key1 >= 0 && rank1 == rho);
-    const int s = b0 ? __builtin_ctzll(b0) : 64 + __builtin_ctzll(b1);
-    it.seq = __builtin_amdgcn_readfirstlane(s);
-    it.ctx = s < 64 ? __builtin_amdgcn_readlane(len0, s) : __builtin_amdgcn_readlane(len1, s - 64);
-    it.c_end = (it.ctx + CT - 1) / CT;
-    it.c_lo = wa.first_visible_chunk(it.ctx, 0);  // the launch's earliest query token decides: the same for both tiles
-    return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
+    if (!items.at(n, G, wg, CT, it)) return false;
+    it.c_lo = wa.first_visible_chunk(it.ctx, it.c_lo);
+    return true;
   };
 
   // Partial states of two items in flight, per column tile: item n goes to buffer n & 1.
@@ -149,7 +104,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     if (lane == 0) __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
-  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, float out_mul) __attribute__((always_inline)) {
+  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, float out_mul) __attribute__((always_inline)) {
     float M = -INFINITY;
 #pragma unroll
     for (int v = 0; v < NW; ++v) M = fmaxf(M, sm_m[tile][b][v][i]);
@@ -173,8 +128,17 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       const int head = kvh * p.group + w.col_g;
       const int d0 = 4 * r * NDT + wave * SL;
       const int64_t row = (int64_t)seq * p.query_len + w.col_q;
-      const float inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key
-      W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
+      const float inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key (of the segment)
+      if constexpr (PART) {
+        const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part0;
+        W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
+        if (r == 0 && wave == 0) {       // one lane per column
+          p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
+          p.exp_sums[slot] = L;
+        }
+      } else {
+        W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
+      }
     }
   };
   // Every wavefront runs  ... finish(n-2), publish(n-1), finish(n-1), publish(n) ...  in this order.
@@ -182,7 +146,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   // later than finish(n-2): the wait ends.  And publish(n) overwrites the buffer of item n-2 only
   // after finish(n-1) has seen every wavefront's publish(n-1), which each of them issues after
   // its finish(n-2).
-  auto finish = [&](int item, int seq, int kvh, float out_mul) __attribute__((always_inline)) {
+  auto finish = [&](int item, const Item &it, float out_mul) __attribute__((always_inline)) {
     const int b = item & 1;
     const int target = NW * ((item >> 1) + 1);
     bool arrived = false;
@@ -196,8 +160,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     }
     if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    finish_tile(wa, 0, b, seq, kvh, out_mul);
-    finish_tile(wb, 1, b, seq, kvh, out_mul);
+    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, out_mul);
+    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, out_mul);
   };
   auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
   // this wavefront's chunks of an item: c_lo + wave, + NW, ... below c_end
@@ -216,14 +180,15 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   Ids ids1 = {};  // block ids of the item's second chunk, requested an item early
   if (m > 0) {
     Ids ids;
+    bool have_ids = false;
+    if constexpr (!PART) {
+      if (cur.c_lo == 0) {  // the ids requested with the lengths are those of chunk `wave`
 #pragma unroll
-    for (int t = 0; t < TPC; ++t) {
-      const int raw = cur.seq < 64 ? __builtin_amdgcn_readlane(sid0[t], cur.seq)
-                                   : __builtin_amdgcn_readlane(sid1[t], cur.seq - 64);
-      ids.v[t] = min((uint32_t)raw, (uint32_t)p.max_block_id);
+        for (int t = 0; t < TPC; ++t) ids.v[t] = min((uint32_t)items.first_id(t, cur.seq), (uint32_t)p.max_block_id);
+        have_ids = true;
+      }
     }
-    if (cur.c_lo != 0)  // the ids requested with the lengths are those of chunk `wave`
-      ids = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave, col_max);
+    if (!have_ids) ids = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave, col_max);
     ids1 = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave + NW, col_max);
     wa.load_q(cur.seq, cur.kvh);
     wb.load_q(cur.seq, cur.kvh);
@@ -231,7 +196,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     wa.issue_v(R0, cur.kvh, cur.c_lo + wave, ids);
     ts0 = wa.fetch_scales(ids, cur.kvh, cur_a);
   }
-  uint32_t sink_a = wa.load_sink(cur.kvh, wave == 0), sink_b = wb.load_sink(cur.kvh, wave == 0);
+  uint32_t sink_a = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0), sink_b = wb.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
   float prev_out_mul = 1.f;
 
@@ -256,15 +221,15 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     wb.set_item(cur_b, cur.ctx);
     uint32_t next_a = W::kNoSink, next_b = W::kNoSink;
     if (has_next && !next_armed) {  // the sink goes with the item whether or not wavefront 0 has a chunk of it
-      next_a = wa.load_sink(nxt.kvh, wave == 0);
-      next_b = wb.load_sink(nxt.kvh, wave == 0);
+      next_a = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      next_b = wb.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
     }
     // What the next item needs beyond K and V, once the last scores of this one are out.
     auto request_next_item = [&]() __attribute__((always_inline)) {
       wa.load_q(nxt.seq, nxt.kvh);
       wb.load_q(nxt.seq, nxt.kvh);
-      next_a = wa.load_sink(nxt.kvh, wave == 0);
-      next_b = wb.load_sink(nxt.kvh, wave == 0);
+      next_a = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      next_b = wb.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
     };
     TileScales nts = {};
     bool owed = n > 0;  // finish(n - 1) still to do
@@ -316,9 +281,9 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
             }
           };
           k_loads(0);
-          const auto pa = wa.template soft<false, true>(X, sa, cx, cur.ctx, &tsx);
+          const auto pa = wa.template soft<false, true>(X, sa, cx, cur.tok_end, &tsx);
           k_loads(1);
-          const auto pb = wb.template soft<false, true>(X, sb, cx, cur.ctx, &tsx);
+          const auto pb = wb.template soft<false, true>(X, sb, cx, cur.tok_end, &tsx);
           k_loads(2);
           W::pv_two(wa, wb, X, pa, pb, [&](int slot) __attribute__((always_inline)) {
             if (slot == W::NP2 * W::NDT / 2 - 1) k_loads(3);
@@ -334,7 +299,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
         while (j + 3 < m) {
           steady(R0, ts0, vp0, R1, vp1, c0 + j * NW, ids_a);
           if (owed) {  // a chunk into the item, the next requests on their way: the merge owed to the item before
-            finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
+            finish(n - 1, prev, prev_out_mul);
             owed = false;
           }
           steady(R1, ts1, vp1, R0, vp0, c0 + (j + 1) * NW, ids_b);
@@ -365,8 +330,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
-        const auto pa = wa.template soft<true, true>(R0, sa, ca, cur.ctx, &ts0);
-        const auto pb = wb.template soft<true, true>(R0, sb, ca, cur.ctx, &ts0);
+        const auto pa = wa.template soft<true, true>(R0, sa, ca, cur.tok_end, &ts0);
+        const auto pb = wb.template soft<true, true>(R0, sb, ca, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
         if (rem == 3) {
           wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
@@ -382,8 +347,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R1, nxt.kvh, nxt.c_lo + wave + NW, nxt_ids1);
           k1_ready = true;
         }
-        const auto pa = wa.template soft<true, true>(R1, sa, ca + NW, cur.ctx, &ts1);
-        const auto pb = wb.template soft<true, true>(R1, sb, ca + NW, cur.ctx, &ts1);
+        const auto pa = wa.template soft<true, true>(R1, sa, ca + NW, cur.tok_end, &ts1);
+        const auto pb = wb.template soft<true, true>(R1, sb, ca + NW, cur.tok_end, &ts1);
         W::pv_two(wa, wb, R1, pa, pb);
       }
       if (rem == 3) {
@@ -393,8 +358,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
-        const auto pa = wa.template soft<true, true>(R0, sa, ca + 2 * NW, cur.ctx, &ts0);
-        const auto pb = wb.template soft<true, true>(R0, sb, ca + 2 * NW, cur.ctx, &ts0);
+        const auto pa = wa.template soft<true, true>(R0, sa, ca + 2 * NW, cur.tok_end, &ts0);
+        const auto pb = wb.template soft<true, true>(R0, sb, ca + 2 * NW, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
         if (next_armed) wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
         ts0 = nts;
@@ -406,7 +371,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
       ts0 = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
     }
-    if (owed) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
+    if (owed) finish(n - 1, prev, prev_out_mul);
     publish(n);
 
     if (!has_next) break;
@@ -421,7 +386,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     cur_b = nxt_b;
     ++n;
   }
-  finish(n, cur.seq, cur.kvh, cur_a.out_mul);
+  finish(n, cur, cur_a.out_mul);
 }
 
 }  // namespace fa
