@@ -48,9 +48,9 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       // sequences first, with the next item's first loads issued before each merge.
       constexpr int PW = PersistentLoop<KV8>::waves;
       auto plain = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                     Pipeline<KV8>::tiles_per_chunk, false, 1, KROW>;
+                                                     Pipeline<KV8>::tiles_per_chunk, false, KROW>;
       auto extended = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                        Pipeline<KV8>::tiles_per_chunk, true, 1, KROW>;
+                                                        Pipeline<KV8>::tiles_per_chunk, true, KROW>;
       // two column tiles in the registers of every wavefront: K and V are loaded once for both
       auto two_tiles = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, PW, TwoTile<KV8>::tiles_per_chunk, KROW>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;

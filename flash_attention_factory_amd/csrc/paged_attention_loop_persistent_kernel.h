@@ -37,18 +37,11 @@ constexpr int kLoopPersistentSpinLimit = 1 << 24;
 constexpr int32_t kStatusSpinLimit = 1;
 
 //
-// TILES (extended instances): column tiles per launch.  The NWG wavefronts of a work-group then
-// form TILES groups of NWG / TILES; every group walks the SAME items and chunks with its own 16
-// (query token, head) columns -- group g holds the query tokens from p.query_first + g * (16 / G)
-// on -- and merges and stores for itself.  The groups run the same code on the same chunks at
-// the same time, so K and V come from HBM once and from the cache for the other groups
-// (their loads are not marked non-temporal for that reason).
-template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, int TILES = 1, bool KROW = true>
+template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, bool KROW = true>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
-  static_assert(TILES == 1 || EXT, "column tiles belong to the extended instances");
-  constexpr int NW = NWG / TILES;  // wavefronts that share an item's chunks and merge: one group
-  using W = WaveAttn<D, QT, KVF, TPC, TILES == 1 && Pipeline<(KVF != 0)>::stream_loads_loop, EXT, KROW>;
+  constexpr int NW = NWG;  // wavefronts that share an item's chunks and merge
+  using W = WaveAttn<D, QT, KVF, TPC, Pipeline<(KVF != 0)>::stream_loads_loop, EXT, KROW>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   using ItemExt = typename W::ItemExt;
@@ -57,12 +50,10 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
   constexpr int SL = NR / NW;
-  static_assert(NWG % TILES == 0 && NW > 1 && NR % NW == 0 && SL >= 2, "merge slices the output across wavefronts");
+  static_assert(NW > 1 && NR % NW == 0 && SL >= 2, "merge slices the output across wavefronts");
 
   const int lane = threadIdx.x & 63;
-  const int wave_of_group = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int tile = TILES > 1 ? wave_of_group / NW : 0;
-  const int wave = TILES > 1 ? wave_of_group % NW : wave_of_group;  // within its group
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int S = p.num_seqs;
   const int Hk = p.num_kv_heads;
   const int T = S * Hk;
@@ -129,12 +120,12 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   };
 
   // Partial states of two items in flight: item n goes to buffer n & 1.
-  __shared__ float sm_m[TILES][2][NW][16];
-  __shared__ float sm_l[TILES][2][NW][16];
-  __shared__ float sm_acc[TILES][2][NW][NR][64];
-  __shared__ int sm_arrived[TILES][2];  // wavefronts of the group that have published into the buffer, ever
+  __shared__ float sm_m[2][NW][16];
+  __shared__ float sm_l[2][NW][16];
+  __shared__ float sm_acc[2][NW][NR][64];
+  __shared__ int sm_arrived[2];  // wavefronts that have published into the buffer, ever
 
-  W wa(p, lane, tile);
+  W wa(p, lane);
   const int r = wa.r, i = wa.i;
   Chunk R;
 
@@ -142,7 +133,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   Item cur;
   if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
   if constexpr (EXT) cur.c_lo = wa.first_visible_chunk(cur.ctx, 0);
-  if (threadIdx.x < 2 * TILES) sm_arrived[threadIdx.x >> 1][threadIdx.x & 1] = 0;
+  if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
   // A wavefront's state of item n goes to LDS and the wavefront moves on; nobody waits here.
@@ -151,14 +142,14 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     wa.settle();
     wa.l = rows_sum(wa.l);
     if (r == 0) {
-      sm_m[tile][b][wave][i] = wa.m;
-      sm_l[tile][b][wave][i] = wa.l;
+      sm_m[b][wave][i] = wa.m;
+      sm_l[b][wave][i] = wa.l;
     }
 #pragma unroll
-    for (int k = 0; k < NR; ++k) sm_acc[tile][b][wave][k][lane] = wa.acc_at(k);
+    for (int k = 0; k < NR; ++k) sm_acc[b][wave][k][lane] = wa.acc_at(k);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     if (lane == 0)
-      __hip_atomic_fetch_add(&sm_arrived[tile][b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of an item, normalise, store this wavefront's slice.
   // Called one chunk into the following item (or after the last item), when the other
@@ -172,7 +163,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     const int target = NW * ((item >> 1) + 1);
     bool arrived = false;
     for (int spin = 0; spin < p.spin_limit; ++spin) {
-      const int seen = __hip_atomic_load(&sm_arrived[tile][b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const int seen = __hip_atomic_load(&sm_arrived[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (__builtin_amdgcn_readfirstlane(seen) >= target) {
         arrived = true;
         break;
@@ -185,21 +176,21 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[tile][b][w][i]);
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[b][w][i]);
     float f[NW];
     float L = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float mw = sm_m[tile][b][w][i];
+      const float mw = sm_m[b][w][i];
       f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
-      L += f[w] * sm_l[tile][b][w][i];
+      L += f[w] * sm_l[b][w][i];
     }
     float o[SL];
 #pragma unroll
     for (int k = 0; k < SL; ++k) {
       float a = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[tile][b][w][wave * SL + k][lane];
+      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + k][lane];
       o[k] = a;
     }
     if (wa.col_valid && wa.keeps_output()) {

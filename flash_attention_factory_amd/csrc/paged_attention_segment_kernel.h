@@ -33,14 +33,11 @@
 namespace fa {
 
 //
-// TILES (extended instances): column tiles per launch, held by TILES groups of NWG / TILES
-// wavefronts that walk the same segments, as in the persistent loop kernel.
-template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, int TILES = 1>
+template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_segment_kernel(const PagedAttnParams p) {
-  static_assert(TILES == 1 || EXT, "column tiles belong to the extended instances");
-  constexpr int NW = NWG / TILES;  // wavefronts that share a segment's chunks and merge: one group
-  using W = WaveAttn<D, QT, KVF, TPC, TILES == 1 && SegmentSplit<(KVF != 0)>::stream_loads, EXT>;
+  constexpr int NW = NWG;  // wavefronts that share a segment's chunks and merge
+  using W = WaveAttn<D, QT, KVF, TPC, SegmentSplit<(KVF != 0)>::stream_loads, EXT>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
   using ItemExt = typename W::ItemExt;
@@ -50,13 +47,11 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   constexpr int NDT = W::NDT;
   constexpr int SL = NR / NW;
   constexpr int NQ = kSegmentMaxSeqs / 64;
-  static_assert(NWG % TILES == 0 && NW > 1 && NR % NW == 0 && SL >= 4 && SL % 4 == 0,
+  static_assert(NW > 1 && NR % NW == 0 && SL >= 4 && SL % 4 == 0,
                 "each wavefront stores whole 16-byte pieces");
 
   const int lane = threadIdx.x & 63;
-  const int wave_of_group = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int tile = TILES > 1 ? wave_of_group / NW : 0;
-  const int wave = TILES > 1 ? wave_of_group % NW : wave_of_group;  // within its group
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int S = p.num_seqs;
   const int Hk = p.num_kv_heads;
   const int G = gridDim.x;
@@ -156,16 +151,16 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   auto position = [&](int nth) { return nth * G + ((nth & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x); };
 
   // Partial states of two items in flight: the n-th item of this work-group goes to buffer n & 1.
-  __shared__ float sm_m[TILES][2][NW][16];
-  __shared__ float sm_l[TILES][2][NW][16];
-  __shared__ float sm_acc[TILES][2][NW][NR][64];
-  __shared__ int sm_arrived[TILES][2];  // wavefronts of the group that have published into the buffer, ever
+  __shared__ float sm_m[2][NW][16];
+  __shared__ float sm_l[2][NW][16];
+  __shared__ float sm_acc[2][NW][NR][64];
+  __shared__ int sm_arrived[2];  // wavefronts that have published into the buffer, ever
 
   if ((int)blockIdx.x >= total_items) return;  // the same for every wavefront of the work-group
-  if (threadIdx.x < 2 * TILES) sm_arrived[threadIdx.x >> 1][threadIdx.x & 1] = 0;
+  if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
-  W wa(p, lane, tile);
+  W wa(p, lane);
   const int r = wa.r, i = wa.i;
   Chunk R;
   // EXT: a segment is read from its first chunk inside the local window
@@ -178,14 +173,14 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     wa.settle();
     wa.l = rows_sum(wa.l);
     if (r == 0) {
-      sm_m[tile][b][wave][i] = wa.m;
-      sm_l[tile][b][wave][i] = wa.l;
+      sm_m[b][wave][i] = wa.m;
+      sm_l[b][wave][i] = wa.l;
     }
 #pragma unroll
-    for (int e = 0; e < NR; ++e) sm_acc[tile][b][wave][e][lane] = wa.acc_at(e);
+    for (int e = 0; e < NR; ++e) sm_acc[b][wave][e][lane] = wa.acc_at(e);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     if (lane == 0)
-      __hip_atomic_fetch_add(&sm_arrived[tile][b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of the work-group's n-th item, normalise, store this
   // wavefront's slice of the partial (see the persistent loop kernel for why the wait
@@ -195,7 +190,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     const int target = NW * ((n >> 1) + 1);
     bool arrived = false;
     for (int spin = 0; spin < p.spin_limit; ++spin) {
-      const int seen = __hip_atomic_load(&sm_arrived[tile][b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const int seen = __hip_atomic_load(&sm_arrived[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (__builtin_amdgcn_readfirstlane(seen) >= target) {
         arrived = true;
         break;
@@ -208,21 +203,21 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[tile][b][w][i]);
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[b][w][i]);
     float f[NW];
     float L = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float mw = sm_m[tile][b][w][i];
+      const float mw = sm_m[b][w][i];
       f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
-      L += f[w] * sm_l[tile][b][w][i];
+      L += f[w] * sm_l[b][w][i];
     }
     float o[SL];
 #pragma unroll
     for (int e = 0; e < SL; ++e) {
       float a = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[tile][b][w][wave * SL + e][lane];
+      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + e][lane];
       o[e] = a;
     }
     if (wa.col_valid && wa.keeps_output()) {
