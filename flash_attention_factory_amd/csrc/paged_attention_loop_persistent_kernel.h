@@ -22,6 +22,7 @@
 // skipped, so an item starts at its first visible chunk.
 #pragma once
 
+#include "paged_attention_items.h"
 #include "paged_attention_kernel.h"
 
 namespace fa {
@@ -54,70 +55,16 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int S = p.num_seqs;
-  const int Hk = p.num_kv_heads;
-  const int T = S * Hk;
   const int G = gridDim.x;
   const int wg = blockIdx.x;
-  const int max_ctx = p.max_blocks_per_seq << p.block_shift;
   const int col_max = p.max_blocks_per_seq - 1;
 
-  // ---- rank the sequences by length, longest first; lane holds sequences lane, lane+64 --
-  // Requested together with the lengths, so that the first K/V loads depend on one round
-  // trip to memory, not two: for EVERY sequence, the block ids of the chunk this wavefront
-  // would start with.  Once the ranking has named the first item its ids are a lane away.
-  int len0 = -1, len1 = -1;
-  int sid0[TPC] = {}, sid1[TPC] = {};
-  if (lane < S) {
-    len0 = max(0, min(p.context_lens[lane], max_ctx));
-    const int32_t *row = p.block_tables + (int64_t)lane * p.max_blocks_per_seq;
-#pragma unroll
-    for (int t = 0; t < TPC; ++t) sid0[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
-  }
-  if (S > 64 && lane + 64 < S) {
-    len1 = max(0, min(p.context_lens[lane + 64], max_ctx));
-    const int32_t *row = p.block_tables + (int64_t)(lane + 64) * p.max_blocks_per_seq;
-#pragma unroll
-    for (int t = 0; t < TPC; ++t) sid1[t] = row[min((wave * CT + t * kTileTokens) >> p.block_shift, col_max)];
-  }
-  // Sort key: length, then lower sequence number first; distinct for distinct sequences
-  // (lengths stay below 2^24, the launcher sees to that).  Lanes without a sequence: -1.
-  const int key0 = len0 < 0 ? -1 : (len0 << 7) | (127 - lane);
-  const int key1 = len1 < 0 ? -1 : (len1 << 7) | (63 - lane);
-  int rank0 = 0, rank1 = 0;  // how many sequences come before this one
-  // eight sequences per trip; lanes past the batch hold -1 and count for nothing
-  for (int u0 = 0; u0 < min(S, 64); u0 += 8) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int ku = __builtin_amdgcn_readlane(key0, u0 + j);
-      rank0 += ku > key0;
-      rank1 += ku > key1;
-    }
-  }
-  for (int u0 = 0; u0 < S - 64; u0 += 8) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int ku = __builtin_amdgcn_readlane(key1, u0 + j);
-      rank0 += ku > key0;
-      rank1 += ku > key1;
-    }
-  }
-  struct Item { int seq, kvh, ctx, c_end, c_lo; };  // c_lo: first chunk to read (0 unless EXT)
-  // n-th item of this work-group: position n*G + j on even n, n*G + G-1-j on odd n
-  auto item_at = [&](int n, Item &it) -> bool {
-    const int pos = n * G + ((n & 1) ? G - 1 - wg : wg);
-    if (pos >= T) return false;
-    const int rho = __builtin_amdgcn_readfirstlane(pos / Hk);
-    it.kvh = pos - rho * Hk;
-    const unsigned long long b0 = __ballot(key0 >= 0 && rank0 == rho);
-    const unsigned long long b1 = __ballot(key1 >= 0 && rank1 == rho);
-    const int s = b0 ? __builtin_ctzll(b0) : 64 + __builtin_ctzll(b1);
-    it.seq = __builtin_amdgcn_readfirstlane(s);
-    it.ctx = s < 64 ? __builtin_amdgcn_readlane(len0, s) : __builtin_amdgcn_readlane(len1, s - 64);
-    it.c_end = (it.ctx + CT - 1) / CT;
-    it.c_lo = 0;
-    return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
-  };
+  // The items, (sequence, kv head) pairs with the longest sequences first, dealt in snake order;
+  // c_lo: first chunk to read (0 unless EXT)
+  using Item = WorkItem;
+  LoopItems<TPC> items;
+  items.build(p, lane, wave, G, CT);
+  auto item_at = [&](int n, Item &it) -> bool { return items.at(n, G, wg, CT, it); };
 
   // Partial states of two items in flight: item n goes to buffer n & 1.
   __shared__ float sm_m[2][NW][16];
@@ -216,9 +163,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     Ids ids;
 #pragma unroll
     for (int t = 0; t < TPC; ++t) {
-      const int raw = cur.seq < 64 ? __builtin_amdgcn_readlane(sid0[t], cur.seq)
-                                   : __builtin_amdgcn_readlane(sid1[t], cur.seq - 64);
-      ids.v[t] = min((uint32_t)raw, (uint32_t)p.max_block_id);
+      ids.v[t] = min((uint32_t)items.first_id(t, cur.seq), (uint32_t)p.max_block_id);
     }
     if constexpr (EXT) {
       if (cur.c_lo != 0)  // the ids requested with the lengths are those of chunk `wave`

@@ -26,6 +26,7 @@
 // sum 0, zeros), which the reduce kernel weighs with 0.
 #pragma once
 
+#include "paged_attention_items.h"
 #include "paged_attention_kernel.h"
 #include "paged_attention_loop_persistent_kernel.h"
 #include "paged_attention_segment_policy.h"
@@ -46,109 +47,22 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
   constexpr int SL = NR / NW;
-  constexpr int NQ = kSegmentMaxSeqs / 64;
   static_assert(NW > 1 && NR % NW == 0 && SL >= 4 && SL % 4 == 0,
                 "each wavefront stores whole 16-byte pieces");
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int S = p.num_seqs;
-  const int Hk = p.num_kv_heads;
   const int G = gridDim.x;
-  const int max_ctx = p.max_blocks_per_seq << p.block_shift;
   const int col_max = p.max_blocks_per_seq - 1;
 
-  // ---- segment list, in registers: lane holds sequences lane, lane+64, ... ---------------
-  // Segments are dealt longest first: all full segments (equal length), then the sequences'
-  // last, shorter segments in order of length; work-group j takes positions j, 2G-1-j,
-  // 2G+j, ... of that list (snake order), so the work-groups' totals come out even although
-  // a work-group only gets a handful of segments.
-  int ctxv[NQ], parts[NQ], incl[NQ], fullc[NQ], key[NQ], rank[NQ];
-  const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size,
-                                               p.max_num_partitions, lane, ctxv, parts);
-  const int m = partitions_per_segment(total_parts, Hk, G);
-  const int seg_tokens = m * p.partition_size;
-  int running = 0, tails = 0;
-#pragma unroll
-  for (int j = 0; j < NQ; ++j) {
-    const int cut = min(ctxv[j], parts[j] * p.partition_size);  // what the scratch arrays can hold
-    ctxv[j] = cut;
-    fullc[j] = cut / seg_tokens;
-    const int rem = cut - fullc[j] * seg_tokens;
-    // sort key of the last segment: length, then lower sequence number first; -1: none
-    key[j] = rem > 0 ? (rem << 8) | (255 - (lane + 64 * j)) : -1;
-    rank[j] = 0;
-    int x = fullc[j];
-    if (j * 64 < S) {
-      tails += __builtin_popcountll(__ballot(rem > 0));
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int y = __shfl_up(x, o);
-        if (lane >= o) x += y;
-      }
-    }
-    incl[j] = x + running;
-    running = __builtin_amdgcn_readlane(incl[j], 63);
-  }
-  const int full_total = running;
-  const int total_items = (full_total + tails) * Hk;
-  // rank of every last segment among the last segments (how many are longer)
-#pragma unroll
-  for (int js = 0; js < NQ; ++js) {
-    if (js * 64 < S) {
-      for (int u0 = 0; u0 < min(S - js * 64, 64); u0 += 8) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int ku = __builtin_amdgcn_readlane(key[js], u0 + e);
-#pragma unroll
-          for (int jd = 0; jd < NQ; ++jd) rank[jd] += ku > key[jd];
-        }
-      }
-    }
-  }
-
-  struct Item { int seq, kvh, part0, tok_end, c_begin, c_end, ctx; };  // ctx: the sequence's length (EXT)
-  // position in the sorted list -> (sequence, segment, kv head), kv head fastest
-  auto decode = [&](int pos) -> Item {
-    Item it;
-    const int q = __builtin_amdgcn_readfirstlane(pos / Hk);
-    it.kvh = pos - q * Hk;
-    int s = 0;
-    const bool full = q < full_total;
-    if (full) {
-#pragma unroll
-      for (int j = 0; j < NQ; ++j)
-        if (j * 64 < S) s += __builtin_popcountll(__ballot(lane + 64 * j < S && incl[j] <= q));
-    } else {
-      const int rho = q - full_total;
-#pragma unroll
-      for (int j = 0; j < NQ; ++j)
-        if (j * 64 < S) {
-          const unsigned long long hit = __ballot(key[j] >= 0 && rank[j] == rho);
-          if (hit) s = 64 * j + __builtin_ctzll(hit);
-        }
-    }
-    s = min(s, S - 1);
-    int inc_s = 0, full_s = 0, ctx_s = 0;
-#pragma unroll
-    for (int j = 0; j < NQ; ++j)
-      if ((s >> 6) == j) {
-        inc_s = __builtin_amdgcn_readlane(incl[j], s & 63);
-        full_s = __builtin_amdgcn_readlane(fullc[j], s & 63);
-        ctx_s = __builtin_amdgcn_readlane(ctxv[j], s & 63);
-      }
-    it.seq = __builtin_amdgcn_readfirstlane(s);
-    const int seg = full ? q - (inc_s - full_s) : full_s;
-    it.part0 = seg * m;
-    const int tok_begin = seg * seg_tokens;
-    it.tok_end = full ? tok_begin + seg_tokens : ctx_s;
-    it.c_begin = tok_begin / CT;
-    it.c_end = (it.tok_end + CT - 1) / CT;
-    it.ctx = ctx_s;
-    return it;
-  };
+  // The segment list (SegmentItems): all full segments, then the sequences' last, shorter segments
+  // in order of length, dealt to the work-groups in snake order, so that the work-groups' totals
+  // come out even although a work-group only gets a handful of segments.
+  using Item = WorkItem;  // c_lo .. c_end: the segment's chunks; ctx: the sequence's length (EXT)
+  SegmentItems items;
+  items.build(p, lane, G);
   // n-th item of this work-group
-  auto position = [&](int nth) { return nth * G + ((nth & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x); };
+  auto item_at = [&](int nth, Item &it) { return items.at(nth, G, (int)blockIdx.x, CT, it); };
 
   // Partial states of two items in flight: the n-th item of this work-group goes to buffer n & 1.
   __shared__ float sm_m[2][NW][16];
@@ -156,7 +70,8 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   __shared__ float sm_acc[2][NW][NR][64];
   __shared__ int sm_arrived[2];  // wavefronts that have published into the buffer, ever
 
-  if ((int)blockIdx.x >= total_items) return;  // the same for every wavefront of the work-group
+  Item cur;
+  if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
   if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
@@ -165,7 +80,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   Chunk R;
   // EXT: a segment is read from its first chunk inside the local window
   auto clip = [&](Item &it) {
-    if constexpr (EXT) it.c_begin = wa.first_visible_chunk(it.ctx, it.c_begin);
+    if constexpr (EXT) it.c_lo = wa.first_visible_chunk(it.ctx, it.c_lo);
   };
 
   auto publish = [&](int n) {
@@ -239,18 +154,17 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   };
 
   int n = 0;
-  Item cur = decode(position(0));
   clip(cur);
   // first chunk of the first item
-  bool armed = cur.c_begin + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  bool armed = cur.c_lo + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
   ItemExt cur_ext = {}, nxt_ext = {};            // extended instances only
   TileScales ts = {}, nts = {}, nxt_ts = {};
   if constexpr (EXT) cur_ext = wa.fetch_item_ext(cur.kvh, p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq);
   if (armed) {
-    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_begin + wave, col_max);
+    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_lo + wave, col_max);
     wa.load_q(cur.seq, cur.kvh);
-    wa.issue_k(R, cur.kvh, cur.c_begin + wave, ids);
-    wa.issue_v(R, cur.kvh, cur.c_begin + wave, ids);
+    wa.issue_k(R, cur.kvh, cur.c_lo + wave, ids);
+    wa.issue_v(R, cur.kvh, cur.c_lo + wave, ids);
     if constexpr (EXT) ts = wa.fetch_scales(ids, cur.kvh, cur_ext);
   }
   uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
@@ -258,19 +172,17 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   float prev_out_mul = 1.f;
 
   while (true) {
-    const int pn = position(n + 1);
-    const bool has_next = pn < total_items;
     Item nxt = cur;
+    const bool has_next = item_at(n + 1, nxt);
     if (has_next) {
-      nxt = decode(pn);
       clip(nxt);
       if constexpr (EXT)
         nxt_ext = wa.fetch_item_ext(nxt.kvh, p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq);
     }
-    const bool next_armed = has_next && nxt.c_begin + wave < nxt.c_end;
+    const bool next_armed = has_next && nxt.c_lo + wave < nxt.c_end;
     Ids nxt_ids = {};
     if (next_armed)
-      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_begin + wave, col_max);
+      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_lo + wave, col_max);
 
     wa.reset(sink_raw);
     if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
@@ -282,7 +194,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;
-      int ci = cur.c_begin + wave;
+      int ci = cur.c_lo + wave;
       Ids nids = wa.fetch_ids(table, ci + NW, col_max);
       if (ci + NW < cur.c_end) {
         {  // first chunk of the item, then the merge owed to the previous item
@@ -319,17 +231,17 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       if (next_armed) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
         next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-        wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+        wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
         if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
       }
       const auto pb = wa.template soft<true, EXT>(R, s, ci, cur.tok_end, &ts);
       wa.pv(R, pb);
-      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
       wa.load_q(nxt.seq, nxt.kvh);
       next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-      wa.issue_k(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
-      wa.issue_v(R, nxt.kvh, nxt.c_begin + wave, nxt_ids);
+      wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
       if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
     if (owed) finish(n - 1, prev, prev_out_mul);
