@@ -29,7 +29,9 @@ reference_perf_recipe  the shape upstream's own perf loop runs (test_paged.py:60
              beside the algorithmic one
 score_modifiers  configuration 1 with soft-capping, ALiBi and a local window switched on
 query_tokens  configuration 1 with four query tokens per sequence (speculative-decoding step);
-             query_tokens_two_tiles: with 32, which fill two tiles of MFMA columns
+             query_tokens_two_tiles: with 32, which fill two tiles of MFMA columns;
+             query_tokens_split_two_tiles: the same in the split path (configurations 2 and 4
+             with 8 and 4 tokens)
 token_major_layout  configurations 1-4 with pools laid out as the reference's tests build them
 kv_block_scales  the FP8 loop configuration with E4M3 pools and per-block K and V scales
 stream_ordered  host cost of a small decode step: blocking `run` calls (upstream's behaviour),
@@ -343,6 +345,40 @@ def _time_query_tokens(built, steps, torch, W, runner, dev, query_len=4):
     return res
 
 
+def _time_query_tokens_split(built, steps, torch, W, runner, dev, query_len):
+    """A split-path configuration with several query tokens per sequence, enough to fill two tiles
+    of MFMA columns (query_len x group > 16): both tiles are held by every wavefront, K and V are
+    read once."""
+    from flash_attention_factory_amd import lib
+    w, ks, vs = built
+    S, H, D = w.query.shape
+    Hk, B = w.num_kv_heads, w.block_size
+    mod = lib.paged_attention_fp8_reduce if w.is_fp8 else lib.paged_attention_reduce
+    query4 = torch.randn((S, query_len, H, D), device=dev).to(w.query.dtype)
+    out4 = torch.zeros_like(query4)
+    NP = max(1, math.ceil(int(w.context_lens.max()) / w.partition_size))
+    ml = torch.zeros((S * query_len, H, NP), dtype=torch.float32, device=dev)
+    es = torch.zeros_like(ml)
+    tmp = torch.zeros((S * query_len, H, NP, D), dtype=torch.float32, device=dev)
+    view = (lambda t: t.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR else (lambda t: t)
+    ts = []
+    for it in range(5 + steps):
+        k = it % len(ks)
+        head = [ml, es, tmp, out4, None, query4, view(ks[k]), view(vs[k]), w.block_tables, w.context_lens, H // Hk, w.scale]
+        if w.is_fp8:
+            head.append(1.0)
+        t = mod.run(*head, B, 0, None, w.sinks, 0.0, partition_size=w.partition_size)
+        if it >= 5:
+            ts.append(t)
+    mean = torch.tensor(ts, dtype=torch.float64).mean(0)
+    us = float(mean.sum())
+    nbytes = w.algorithmic_bytes() + 2 * S * (query_len - 1) * H * D * 2
+    return dict(workload=f"{w.name} with {query_len} query tokens per sequence, causal",
+                kernel="paged_attn_loop_two_tile_kernel<split path> + paged_attn_reduce_kernel",
+                steps=steps, kernel_us_mean=[float(x) for x in mean], us_per_call=us, algorithmic_bytes=nbytes,
+                gbps_kernels=nbytes / us / 1e3, hbm_frac=nbytes / us / 1e3 / HBM_PEAK_GBPS)
+
+
 def _time_block_scales(built, steps, torch, W, runner, dev):
     """The FP8 loop configuration with E4M3 pools and one K and one V scale per physical block
     and kv head (two more fp32 per 16-token tile of 4 KiB)."""
@@ -517,6 +553,10 @@ def main():
         # 32 tokens of one head are two column tiles, both held by every wavefront
         line["query_tokens_two_tiles"] = _time_query_tokens(built[1], max(20, args.steps // 2), torch, W, runner, dev,
                                                             query_len=32)
+        # the split path with two tiles: 8 tokens x 4 heads of config 2, 4 tokens x 8 heads of config 4
+        line["query_tokens_split_two_tiles"] = [
+            _time_query_tokens_split(built[idx], sub_steps, torch, W, runner, dev, ql)
+            for idx, ql in ((2, 8), (4, 4)) if idx in built]
         # the FP8 loop configuration once more with E4M3 bytes in the pools (same shape, same bytes moved)
         e4m3 = _build_config(3, torch, W, runner, dev, fp8_dtype=torch.float8_e4m3fn)
         _, r = _time_config(e4m3, max(20, args.steps // 2), args.warmup, torch, W, runner, dev)
