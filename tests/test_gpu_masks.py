@@ -258,6 +258,44 @@ def test_more_query_tokens_than_the_mfma_columns_hold(oracle, QL, nheads, nheads
         assert_close_to_reference(got, ref, f"{kernel} QL={QL}")
 
 
+@pytest.mark.parametrize("fp8,qdtype,block_scales", [(False, torch.float16, False), (True, torch.bfloat16, False),
+                                                      (True, torch.float16, True)])
+def test_two_tile_kernels_at_the_edges_of_their_item_lists(oracle, fp8, qdtype, block_scales):
+    """Two column tiles (2 heads x 16 tokens) over 100 sequences -- more than the 64 a wavefront's
+    lanes hold at once -- whose lengths give a wavefront every number of chunks from none to a few
+    more than the steady loop needs: 0, less than the query block, 1 .. 5 chunks of 32 tokens per
+    wavefront with and without a ragged end, on and one past partition and chunk boundaries.  With
+    soft-capping, a window and sinks; with per-block FP8 scales in the third case.  Both paths."""
+    S, QL, H, Hk, D = 100, 16, 4, 2, 128
+    edge = [0, 5, 16, 17, 31, 32, 33, 127, 128, 129, 160, 255, 256, 257, 384, 385, 500, 511, 512, 513, 640, 641, 700,
+            768, 769, 896, 1000, 1023, 1024, 1025, 1100]
+    w = W.make_test_shaped(batch_size=S, nheads=H, nheads_k=Hk, d=D, seqlen_k=1100, varlen=False, has_sinks=True,
+                           fp8=fp8, block_size=16, seed=23, dtype=qdtype)
+    w.context_lens = torch.tensor([edge[(7 * s) % len(edge)] for s in range(S)], dtype=torch.int32)
+    w.sinks = torch.linspace(-2, 2, H).to(qdtype)
+    g = torch.Generator().manual_seed(9)
+    query4 = torch.randn(S, QL, H, D, generator=g).to(qdtype)
+    kw, okw = {}, {}
+    if block_scales:
+        NB = w.key_cache.shape[0]
+        ks = (torch.rand(NB, Hk, generator=g) * 1.5 + 0.5).float()
+        vs = (torch.rand(NB, Hk, generator=g) * 1.5 + 0.5).float()
+        okw = dict(k_scales=ks, v_scales=vs)
+        kw = dict(k_scales=ks.to(_dev()), v_scales=vs.to(_dev()))
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, fp8_scale=w.fp8_scale, want_f32=True, softcap=15.0, window_left=600,
+                               **okw)[1]
+    wd = w.to(_dev())
+    live = w.context_lens > 0
+    for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+        got = _call_multi(wd, query4.to(_dev()), kernel, softcap=15.0, apply_softcap=True, window_left=600,
+                          **kw).float().cpu()
+        assert torch.isfinite(got).all(), kernel
+        assert (got[~live] == 0).all(), kernel          # empty sequences: rows untouched
+        assert_close_to_reference(got[live], ref[live], f"{kernel} fp8={fp8} block_scales={block_scales}")
+
+
 @pytest.mark.parametrize("index,QL", [(4, 4), (1, 32), (2, 8)])
 def test_full_size_query_blocks_with_modifiers(oracle, index, QL):
     """The measured configurations at full size with a query block of two column tiles (G x QL =
