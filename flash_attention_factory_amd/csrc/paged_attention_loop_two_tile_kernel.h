@@ -281,9 +281,9 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
             }
           };
           k_loads(0);
-          const auto pa = wa.template soft<false, true>(X, sa, cx, cur.tok_end, &tsx);
+          const auto pa = wa.template soft<false, true, true>(X, sa, cx, cur.tok_end, &tsx);
           k_loads(1);
-          const auto pb = wb.template soft<false, true>(X, sb, cx, cur.tok_end, &tsx);
+          const auto pb = wb.template soft<false, true, true>(X, sb, cx, cur.tok_end, &tsx);
           k_loads(2);
           W::pv_two(wa, wb, X, pa, pb, [&](int slot) __attribute__((always_inline)) {
             if (slot == W::NP2 * W::NDT / 2 - 1) k_loads(3);
@@ -330,8 +330,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
-        const auto pa = wa.template soft<true, true>(R0, sa, ca, cur.tok_end, &ts0);
-        const auto pb = wb.template soft<true, true>(R0, sb, ca, cur.tok_end, &ts0);
+        const auto pa = wa.template soft<true, true, true>(R0, sa, ca, cur.tok_end, &ts0);
+        const auto pb = wb.template soft<true, true, true>(R0, sb, ca, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
         if (rem == 3) {
           wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
@@ -347,8 +347,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R1, nxt.kvh, nxt.c_lo + wave + NW, nxt_ids1);
           k1_ready = true;
         }
-        const auto pa = wa.template soft<true, true>(R1, sa, ca + NW, cur.tok_end, &ts1);
-        const auto pb = wb.template soft<true, true>(R1, sb, ca + NW, cur.tok_end, &ts1);
+        const auto pa = wa.template soft<true, true, true>(R1, sa, ca + NW, cur.tok_end, &ts1);
+        const auto pb = wb.template soft<true, true, true>(R1, sb, ca + NW, cur.tok_end, &ts1);
         W::pv_two(wa, wb, R1, pa, pb);
       }
       if (rem == 3) {
@@ -358,8 +358,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
-        const auto pa = wa.template soft<true, true>(R0, sa, ca + 2 * NW, cur.tok_end, &ts0);
-        const auto pb = wb.template soft<true, true>(R0, sb, ca + 2 * NW, cur.tok_end, &ts0);
+        const auto pa = wa.template soft<true, true, true>(R0, sa, ca + 2 * NW, cur.tok_end, &ts0);
+        const auto pb = wb.template soft<true, true, true>(R0, sb, ca + 2 * NW, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
         if (next_armed) wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
         ts0 = nts;

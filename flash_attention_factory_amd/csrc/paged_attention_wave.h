@@ -458,7 +458,11 @@ struct WaveAttn {
   // MASKS (EXT instances): apply the score modifiers p.mask_flags names -- soft-capping, local
   // window, ALiBi, in that order (upstream test_paged.py:92-110) -- and the causal rule, all
   // relative to the position col_last of this column's query token.
-  template <bool CHECK_TAIL, bool MASKS = false>
+  // ACC_IN_AGPRS: the kernel holds more than 256 registers and its accumulators live in AGPRs.
+  // The rarely taken rescale branch then reads them with v_accvgpr_read_b32 spelled out and pins the
+  // results to AGPRs again; left to itself the compiler copies every accumulator to a VGPR in front
+  // of the branch, in every chunk, for the branch's benefit.
+  template <bool CHECK_TAIL, bool MASKS = false, bool ACC_IN_AGPRS = false>
   __device__ __forceinline__ Probs soft(Chunk &R, const Scores &s, int ci, int tok_end,
                                         const TileScales *ts = nullptr) {
     constexpr int NT = 4 * TPC;  // this lane's tokens in the chunk: tile e/4, row 4r + e%4
@@ -526,8 +530,26 @@ struct WaveAttn {
         const float m_to = (MASKS && mt == -INFINITY) ? 0.f : mt;
         const float alpha = fast_exp2(m - m_to);  // exp2(-inf) = 0 for a column that has seen nothing so far
         l *= alpha;
+        if constexpr (ACC_IN_AGPRS) {
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+          for (int dt = 0; dt < NDT; ++dt) {
+            f32x4 t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // Read where it is used: a plain read is hoisted in front of the branch.  (The MFMAs that
+              // wrote these registers, P.V of the chunk before, lie a whole score pass back: no MFMA
+              // result is still on its way.)
+              float x;
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[dt][e]));
+              t[e] = x * alpha;
+            }
+            acc[dt] = t;
+            asm volatile("" : "+a"(acc[dt]));
+          }
+        } else {
+#pragma unroll
+          for (int dt = 0; dt < NDT; ++dt) acc[dt] *= alpha;
+        }
       }
       m = mt;
     }
