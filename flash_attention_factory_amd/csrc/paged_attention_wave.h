@@ -563,11 +563,13 @@ struct WaveAttn {
     l += ps;
     // k-slots (r, e) of step pr = this lane's eight tokens of the step, rounded to the q
     // dtype (paged_attention_kernel_loop.hpp:404-407)
-    if constexpr (MASKS && KV8) {  // per-block V scales ride on the probabilities (1.0 otherwise)
-      // by select: a tile past the context takes its block id from a clamped or unused table
-      // column, and the scale of a block nobody wrote may be anything, NaN included
+    if constexpr (MASKS && KV8) {  // per-block V scales ride on the probabilities
+      if (p.kv_scale_mode == kScaleBlock) {
+        // by select: a tile past the context takes its block id from a clamped or unused table
+        // column, and the scale of a block nobody wrote may be anything, NaN included
 #pragma unroll
-      for (int e = 0; e < NT; ++e) t[e] = t[e] == 0.f ? 0.f : t[e] * ts->v[e >> 2];
+        for (int e = 0; e < NT; ++e) t[e] = t[e] == 0.f ? 0.f : t[e] * ts->v[e >> 2];
+      }
     }
     Probs pb;
 #pragma unroll
