@@ -77,6 +77,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   // Partial states of two items in flight, per column tile: item n goes to buffer n & 1.
   __shared__ float sm_m[2][2][NW][16];
   __shared__ float sm_l[2][2][NW][16];
+  __shared__ float sm_mt[PART ? 2 : 1][2][NW][16];  // true maxima (split path: max_logits)
   __shared__ float sm_acc[2][2][NW][NR][64];
   __shared__ int sm_arrived[2];  // wavefronts that have published (both tiles) into the buffer, ever
 
@@ -86,12 +87,15 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
   // A wavefront's states of item n go to LDS and the wavefront moves on; nobody waits here.
+  // The states go out as they are, sums and accumulators against the reference maximum m, which may
+  // lag the true one (mt): a pass over 64 accumulators in AGPRs to bring them up (WaveAttn::settle)
+  // would cost more than everything else here, and the merge is indifferent to the reference.
   auto publish_tile = [&](W &w, int tile, int b) __attribute__((always_inline)) {
-    w.settle();
     w.l = rows_sum(w.l);
     if (r == 0) {
       sm_m[tile][b][wave][i] = w.m;
       sm_l[tile][b][wave][i] = w.l;
+      if constexpr (PART) sm_mt[tile][b][wave][i] = w.mt;
     }
 #pragma unroll
     for (int k = 0; k < NR; ++k) sm_acc[tile][b][wave][k][lane] = w.acc_at(k);
@@ -132,9 +136,12 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       if constexpr (PART) {
         const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part0;
         W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
-        if (r == 0 && wave == 0) {       // one lane per column
-          p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
-          p.exp_sums[slot] = L;
+        if (r == 0 && wave == 0) {  // one lane per column: the true maximum, and the sum against it
+          float MT = -INFINITY;
+#pragma unroll
+          for (int v = 0; v < NW; ++v) MT = fmaxf(MT, sm_mt[tile][b][v][i]);
+          p.max_logits[slot] = MT * kLn2;  // natural-log units, as upstream stores them
+          p.exp_sums[slot] = MT == -INFINITY ? 0.f : L * fast_exp2(M - MT);
         }
       } else {
         W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
