@@ -292,6 +292,7 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.kv_block_bytes = s.kv_block_stride * r.kv_elem_bytes;
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;
+  p.compute_units = 0;  // the split path's launcher fills it in
   p.pair_heads = 0;
   if (r.pair_heads) {  // the kernel sees pairs of kv heads: half as many, twice the group, rows of two heads
     p.pair_heads = 1;
@@ -305,8 +306,9 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
 // How many work-groups of `threads` threads of a kernel the current device keeps resident
 // (compute units x work-groups per compute unit).  Asked once per (kernel, device); all
 // kernels here share one function-pointer type, so the cache is keyed by the pointer value.
-inline hipError_t resident_groups(void (*kernel)(PagedAttnParams), int threads, int *out) {
-  struct Entry { const void *fn; int dev; int groups; };
+// cus_out, if given: the compute units of the device.
+inline hipError_t resident_groups(void (*kernel)(PagedAttnParams), int threads, int *out, int *cus_out = nullptr) {
+  struct Entry { const void *fn; int dev; int groups; int cus; };
   constexpr int kSlots = 64;
   static thread_local Entry cache[kSlots];
   static thread_local int used = 0;
@@ -317,6 +319,7 @@ inline hipError_t resident_groups(void (*kernel)(PagedAttnParams), int threads, 
   for (int k = 0; k < used; ++k)
     if (cache[k].fn == fn && cache[k].dev == dev) {
       *out = cache[k].groups;
+      if (cus_out) *cus_out = cache[k].cus;
       return hipSuccess;
     }
   int cus = 0, per_cu = 0;
@@ -325,8 +328,9 @@ inline hipError_t resident_groups(void (*kernel)(PagedAttnParams), int threads, 
   e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
   if (e != hipSuccess) return e;
   const int groups = cus * (per_cu > 0 ? per_cu : 1);
-  if (used < kSlots) cache[used++] = Entry{fn, dev, groups};
+  if (used < kSlots) cache[used++] = Entry{fn, dev, groups, cus};
   *out = groups;
+  if (cus_out) *cus_out = cus;
   return hipSuccess;
 }
 

@@ -64,8 +64,9 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
       if (q0 == 0) {
         // Every launch of the call gets the same number of work-groups: the segment length, which
         // the reduce kernel works out again, follows from it.
-        int resident = 0;
-        FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident));
+        int resident = 0, cus = 0;
+        FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident, &cus));
+        p.compute_units = cus;
         if (ext && r.query_len > per_launch && r.query_len % per_launch <= per_tile) {  // a one-tile launch ends the call
           int other = 0;
           FA_HIP_CHECK(resident_groups(extended, SW * 64, &other));

@@ -142,6 +142,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           for (int v = 0; v < NW; ++v) MT = fmaxf(MT, sm_mt[tile][b][v][i]);
           p.max_logits[slot] = MT * kLn2;  // natural-log units, as upstream stores them
           p.exp_sums[slot] = MT == -INFINITY ? 0.f : L * fast_exp2(M - MT);
+          // the row's first segment tells the reduce kernel how long segments are (segment_mark)
+          if (part0 == 0 && items.m > 1 && p.max_num_partitions > 1) p.max_logits[slot + 1] = segment_mark(items.m);
         }
       } else {
         W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);

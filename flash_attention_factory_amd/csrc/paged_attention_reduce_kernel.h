@@ -36,9 +36,9 @@ struct ReduceParams {
   int32_t num_seqs;
   int32_t num_kv_heads;
   int32_t query_len;       // query tokens per sequence: rows of out / scratch are (sequence, query token) pairs
-  int32_t segment_groups;  // work-groups of the segment attention kernel that wrote the partials
-                           // (it wrote one partial per segment of m partitions, into the
-                           // segment's first slot); 0: one partial per partition
+  int32_t segment_groups;  // > 0: a segment attention kernel wrote the partials (one per segment of
+                           // m partitions, into the segment's first slot, and m into slot 1 of
+                           // max_logits: segment_mark); 0: one partial per partition
 };
 
 // Rows requested per wavefront and batch: 16 when every partition has a partial (dozens per
@@ -61,21 +61,23 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   // sequence, or a (sequence, query token) pair
   const int seq = blockIdx.x / p.num_heads;
   const int head = blockIdx.x - seq * p.num_heads;
+  const int64_t base = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions;
+  // Partials lie `stride` slots apart: 1, or the segment length the attention kernel chose and left
+  // in slot 1 of the row (segment_mark).  Requested together with the length, whether or not the
+  // row turns out to have a second partition, so that one wait covers both.
+  float slot1 = 0.f;
+  if constexpr (SEGMENTS) {
+    if (p.max_num_partitions > 1) slot1 = p.max_logits[base + 1];
+  }
   const int ctx = min(p.context_lens[p.query_len > 1 ? seq / p.query_len : seq], p.max_context);
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;
   np = min(np, p.max_num_partitions);
-  // Partials lie `stride` slots apart: 1, or the segment length the attention kernel chose.
   int stride = 1;
   if constexpr (SEGMENTS) {
-    constexpr int NQ = kSegmentMaxSeqs / 64;
-    int ctxv[NQ], parts[NQ];
-    const int total = count_partitions<NQ>(p.context_lens, p.num_seqs, p.max_context, p.partition_size,
-                                           p.max_num_partitions, lane, ctxv, parts);
-    stride = partitions_per_segment(total, p.num_kv_heads, p.segment_groups);
+    if (np > 1) stride = __builtin_amdgcn_readfirstlane(segment_length_of(slot1));
     np = (np + stride - 1) / stride;  // from here on: the number of partials
   }
-  const int64_t base = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions;
   const float *ml = p.max_logits + base;
   const float *es = p.exp_sums + base;
   const float *tmp = p.tmp_out + base * D + lane * EPL;

@@ -1,7 +1,9 @@
-// How the segment form of the split path cuts sequences: shared by the attention kernel
-// that writes one partial per segment (paged_attention_segment_kernel.h) and the reduce
-// kernel that reads them (paged_attention_reduce_kernel.h) -- both evaluate the same
-// function on the same context lengths, so they agree on where the partials lie.
+// How the segment form of the split path cuts sequences.  The attention kernels
+// (paged_attention_segment_kernel.h, the split form of paged_attention_loop_two_tile_kernel.h)
+// choose the segment length from the batch, every wavefront for itself, and write one partial per
+// segment into the slot of the segment's first partition; the reduce kernel
+// (paged_attention_reduce_kernel.h) finds the length in the scratch arrays: a length other than 1
+// leaves slot 1 of every row free, and there the attention kernel leaves a mark (segment_mark).
 #pragma once
 
 #include "paged_attention_utils.h"
@@ -10,48 +12,183 @@ namespace fa {
 
 constexpr int kSegmentMaxSeqs = 256;
 constexpr int kSegmentMaxContext = 1 << 23;  // lengths are packed into 23 bits of a sort key
-// Segments aimed at per resident work-group, and the most partitions one may span.  Measured
-// on the long-context and the serving-mix configurations: 2 beats 1 (the long-context batch
-// loses 12 %), 3, 4 and 8 (the serving mix loses 3, 15 and 16 %: every segment costs a
-// merge, a scattered partial and a restart of the stream).
-#ifndef FA_SEGMENT_ITEMS
-#define FA_SEGMENT_ITEMS 2
-#endif
+// The most partitions one segment may span.
 #ifndef FA_SEGMENT_MAX_PARTS
 #define FA_SEGMENT_MAX_PARTS 64
 #endif
-constexpr int kSegmentItemsPerGroup = FA_SEGMENT_ITEMS;
 constexpr int kSegmentMaxPartitions = FA_SEGMENT_MAX_PARTS;
 
-// How many partitions one segment spans.  total_partitions: live partitions of all
-// sequences; groups: work-groups of the attention launch.
-__device__ __forceinline__ int partitions_per_segment(int total_partitions, int num_kv_heads, int groups) {
-  const long long items = (long long)total_partitions * num_kv_heads;
-  const long long m = items / ((long long)kSegmentItemsPerGroup * max(groups, 1));
-  return (int)max(1LL, min(m, (long long)kSegmentMaxPartitions));
+// a / b for 0 <= a < 2^24 and b >= 1, given inv_b close to 1 / b: both are exact in fp32, so the
+// product is off by one at most, which the remainder tells.
+__device__ __forceinline__ int quotient_below_2p24(int a, int b, float inv_b, int &rem) {
+  int q = (int)((float)a * inv_b);
+  rem = a - q * b;
+  if (rem < 0) { --q; rem += b; }
+  if (rem >= b) { ++q; rem -= b; }
+  return q;
 }
 
-// Live partitions of all sequences, as every wavefront of either kernel computes them:
+// Sum over the 64 lanes of a wavefront (all of them active), in data-parallel-primitive moves
+// rather than trips through the LDS crossbar: the callers run once per wavefront, before the
+// first load of a launch, where every cycle is latency.
+__device__ __forceinline__ int wave_total(int v) {
+  return __builtin_amdgcn_readfirstlane(__reduce_add_sync(~0ull, v));
+}
+
+// Segment length as a share (in 1/1024) of a compute unit's mean load, against the sequences
+// per compute unit (in 1/1024).  Every sequence ends in a segment shorter than the others, so
+// with many sequences per compute unit the short ones alone fill the GPU and only sequences well
+// above the mean are worth cutting; with few, the whole segments are the work and one of them
+// should be what a work-group gets.  Measured on 27 batches of 1 to 256 sequences (the length
+// that was fastest for each, to within a few per cent): 1.12 of the load up to one sequence per
+// compute unit, 0.57 at two, 0.37 at four, 0.35 from eight on.
+__device__ __forceinline__ int segment_share_of_load(int seqs_per_cu_1024) {
+  // straight lines between the measured points; literals and shifts, so that nothing here is a
+  // table in memory or a division
+  const int x = seqs_per_cu_1024;
+  if (x <= 1024) return 1147;
+  if (x <= 2048) return 1147 - ((563 * (x - 1024)) >> 10);
+  if (x <= 4096) return 584 - ((205 * (x - 2048)) >> 11);
+  if (x <= 8192) return 379 - ((19 * (x - 4096)) >> 12);
+  return 360;
+}
+
+// The mark in max_logits[row][1]: a NaN no maximum can be (maxima are finite or -inf, and a NaN
+// that arithmetic makes has none of the low mantissa bits set), the segment length in its low
+// byte.  Rows of one partition need none; with a segment length of 1 slot 1 holds a partial.
+constexpr uint32_t kSegmentMarkBits = 0x7FD3A600u, kSegmentMarkMask = 0xFFFFFF00u;
+static_assert(kSegmentMaxPartitions < 256, "the segment length is kept in one byte of the mark");
+__device__ __forceinline__ float segment_mark(int m) { return __uint_as_float(kSegmentMarkBits | (uint32_t)m); }
+// segment length a row's slot 1 tells: 1 unless it holds the mark
+__device__ __forceinline__ int segment_length_of(float slot1) {
+  const uint32_t bits = __float_as_uint(slot1);
+  if ((bits & kSegmentMarkMask) != kSegmentMarkBits) return 1;
+  return max(1, min((int)(bits & 0xFFu), kSegmentMaxPartitions));
+}
+
+// Whole segments and segments in all (per kv head) that a segment length of m partitions
+// leaves: lane holds sequences lane, lane + 64, ... of which ctxv / parts are the lengths and
+// live partitions.
+template <int NQ>
+__device__ __forceinline__ void count_segments(const int (&ctxv)[NQ], const int (&parts)[NQ], int S,
+                                               int partition_size, int m, int &whole, int &all) {
+  const int seg_tokens = m * partition_size;
+  const float inv = __builtin_amdgcn_rcpf((float)seg_tokens);
+  int f = 0, t = 0;
+#pragma unroll
+  for (int j = 0; j < NQ; ++j)
+    if (j * 64 < S) {  // wave-uniform
+      const int cut = min(ctxv[j], parts[j] * partition_size);  // what the scratch arrays can hold
+      int rem;
+      f += quotient_below_2p24(cut, seg_tokens, inv, rem);  // lengths stay below 2^23 (kSegmentMaxContext)
+      t += __builtin_popcountll(__ballot(rem > 0));
+    }
+  whole = wave_total(f);
+  all = whole + t;
+}
+
+// How many partitions one segment spans, as every wavefront of an attention launch works it out
+// from the same context lengths.  total_partitions: live partitions of all sequences
+// (count_partitions); groups: work-groups of the launch; cus: compute units of the GPU.
+//
+// Work-groups g and g + cus share a compute unit, and what a compute unit streams is what
+// bounds the launch: the length aims at a share of the mean load of a compute unit
+// (segment_share_of_load), or at the mean load of a work-group where several share one and the
+// whole segments are the work.  Whole segments are all of one length, and where they pile up
+// that length is what the launch waits for; so: with few sequences on shared units, one segment
+// per unit if that fits (phase 0 below); else no more whole segments than work-groups (the
+// length grows until that holds), and, with two work-groups per compute unit, not a count of
+// segments between one per unit and most of the work-groups (some units would hold two and
+// stream twice as long as the others; the length grows until every unit holds one).
+template <int NQ>
+__device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], const int (&parts)[NQ],
+                                                      int total_partitions, int S, int partition_size,
+                                                      int num_kv_heads, int groups, int cus) {
+  const int units = max(1, min(groups, cus));  // compute units at work
+  const int sharing = groups <= units ? 1 : groups <= 2 * units ? 2 : (groups + units - 1) / units;  // work-groups on each
+  int live = 0;
+#pragma unroll
+  for (int j = 0; j < NQ; ++j)
+    if (j * 64 < S) live += __builtin_popcountll(__ballot(parts[j] > 0));
+  const float items = (float)total_partitions * (float)num_kv_heads;
+  const float per_unit = __builtin_amdgcn_rcpf((float)units);
+  const float seqs_per_cu = fminf((float)live * (float)num_kv_heads * per_unit, 1024.f);
+  int share = segment_share_of_load((int)(seqs_per_cu * 1024.f));
+  if (sharing > 1) share = min(share, sharing == 2 ? 512 : 1024 / sharing);
+  int m = (int)fminf(items * per_unit * ((float)share * (1.0f / 1024.f)) + 0.5f, (float)kSegmentMaxPartitions);
+  m = max(m, 1);
+  if (m == 1 && items <= (float)groups) return 1;  // a partition per work-group at most: nothing to weigh
+  // Few sequences on shared compute units: first try one segment per unit (the shortest length
+  // that leaves no more segments than units), as long as a segment is then at most 1.25 of a
+  // unit's mean load -- a work-group alone on its unit streams that much faster than its share.
+  const long long items_all = (long long)total_partitions * num_kv_heads;
+  const bool few = sharing > 1 && 2 * live * num_kv_heads <= units;
+  const int aimed = m;
+  int phase = 1;  // 0: one segment per unit; 1: no more whole segments than work-groups; 2: not between
+  if (few && items_all > units) {
+    phase = 0;
+    m = (int)fminf(ceilf(items * per_unit), (float)kSegmentMaxPartitions);
+  }
+  // One loop, not unrolled: this code runs once per wavefront, at the speed instructions arrive
+  // from memory, so its size is its cost.
+  int before = 0, tries = 0;
+#pragma nounroll
+  for (int evaluations = 0; evaluations < 12; ++evaluations) {
+    if (phase == 0 && (tries >= 4 || m > kSegmentMaxPartitions || 4LL * m * units > 5 * items_all)) {
+      phase = 1;
+      m = aimed;
+      tries = 0;
+    }
+    int whole, all;
+    count_segments<NQ>(ctxv, parts, S, partition_size, m, whole, all);
+    const long long n = (long long)all * num_kv_heads;
+    if (phase == 0) {
+      if (n <= units) return m;
+      ++m;
+      ++tries;
+      continue;
+    }
+    if (phase == 1) {
+      if ((long long)whole * num_kv_heads > groups && tries < 3 && m < kSegmentMaxPartitions) {
+        ++m;
+        ++tries;
+        continue;
+      }
+      if (!(few && n > units && n * 20 < (long long)groups * 17)) return m;
+      phase = 2;
+      before = m;
+    } else if (n <= units) {
+      return m;
+    }
+    if (m - before >= 4 || m >= kSegmentMaxPartitions) return before;
+    ++m;
+  }
+  return before > 0 ? before : m;
+}
+
+// Live partitions of all sequences, as every wavefront of an attention launch computes them:
 // lane holds sequences lane, lane+64, ...  Returns the total; per-lane counts in `parts`.
 template <int NQ>
 __device__ __forceinline__ int count_partitions(const int32_t *context_lens, int S, int max_ctx,
                                                 int partition_size, int max_num_partitions, int lane,
                                                 int (&ctxv)[NQ], int (&parts)[NQ]) {
+  // every lane asks for its NQ lengths at once (lanes past the batch for the last one, which they
+  // then drop): one trip to memory, not one per 64 sequences
+  int len[NQ];
+#pragma unroll
+  for (int j = 0; j < NQ; ++j) len[j] = context_lens[min(lane + 64 * j, S - 1)];
   int local = 0;
+  const float inv = __builtin_amdgcn_rcpf((float)partition_size);
 #pragma unroll
   for (int j = 0; j < NQ; ++j) {
-    const int s = lane + 64 * j;
-    int c = 0;
-    if (j * 64 < S) {  // wave-uniform
-      if (s < S) c = max(0, min(context_lens[s], max_ctx));
-    }
+    const int c = lane + 64 * j < S ? max(0, min(len[j], max_ctx)) : 0;
     ctxv[j] = c;
-    parts[j] = min((c + partition_size - 1) / partition_size, max_num_partitions);
+    // lengths and the partition size stay below 2^23 (kSegmentMaxContext: the launcher sees to it)
+    int rem;
+    parts[j] = min(quotient_below_2p24(c + partition_size - 1, partition_size, inv, rem), max_num_partitions);
     local += parts[j];
   }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) local += __shfl_xor(local, o);
-  return __builtin_amdgcn_readfirstlane(local);
+  return wave_total(local);
 }
 
 }  // namespace fa

@@ -78,6 +78,9 @@ struct PagedAttnParams {
   // kv_head_bytes describe the pairs -- while query and out rows keep 64 elements.  See
   // WaveAttn::kPairable.
   int32_t pair_heads;
+  // compute units of the GPU: the split path's segment length depends on it
+  // (partitions_per_segment)
+  int32_t compute_units;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
