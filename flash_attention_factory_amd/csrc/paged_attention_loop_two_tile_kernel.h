@@ -108,7 +108,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     if (lane == 0) __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
-  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, float out_mul) __attribute__((always_inline)) {
+  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool mark, float out_mul) __attribute__((always_inline)) {
     float M = -INFINITY;
 #pragma unroll
     for (int v = 0; v < NW; ++v) M = fmaxf(M, sm_m[tile][b][v][i]);
@@ -142,8 +142,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           for (int v = 0; v < NW; ++v) MT = fmaxf(MT, sm_mt[tile][b][v][i]);
           p.max_logits[slot] = MT * kLn2;  // natural-log units, as upstream stores them
           p.exp_sums[slot] = MT == -INFINITY ? 0.f : L * fast_exp2(M - MT);
-          // the row's first segment tells the reduce kernel how long segments are (segment_mark)
-          if (part0 == 0 && items.m > 1 && p.max_num_partitions > 1) p.max_logits[slot + 1] = segment_mark(items.m);
+          if (mark) p.max_logits[slot + 1] = segment_mark(items.m);  // for the reduce kernel
         }
       } else {
         W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
@@ -169,8 +168,11 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     }
     if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, out_mul);
-    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, out_mul);
+    // a row of two or more partitions: its first segment leaves the segment length (segment_mark)
+    bool mark = false;
+    if constexpr (PART) mark = it.part0 == 0 && items.m > 1 && it.ctx > p.partition_size && p.max_num_partitions > 1;
+    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, mark, out_mul);
+    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, mark, out_mul);
   };
   auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
   // this wavefront's chunks of an item: c_lo + wave, + NW, ... below c_end

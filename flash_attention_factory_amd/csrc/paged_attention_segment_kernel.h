@@ -149,8 +149,10 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       if ((wa.paired() ? (r & 1) == 0 : r == 0) && wave == 0) {  // one lane per column, see merge_and_store
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;
-        // the row's first segment tells the reduce kernel how long segments are (segment_mark)
-        if (it.part0 == 0 && items.m > 1 && p.max_num_partitions > 1) p.max_logits[slot + 1] = segment_mark(items.m);
+        // the first segment of a row of two or more partitions tells the reduce kernel how long
+        // segments are (segment_mark)
+        if (it.part0 == 0 && items.m > 1 && it.ctx > p.partition_size && p.max_num_partitions > 1)
+          p.max_logits[slot + 1] = segment_mark(items.m);
       }
     }
   };

@@ -223,21 +223,39 @@ def test_persistent_split_many_items_per_wavefront(oracle):
     torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
 
 
-def test_segment_kernel_partials_lie_a_segment_apart(oracle):
-    """A batch with enough (sequence, kv head) pairs that the split path works in segments of
-    several partitions: the output matches the oracle, and the scratch arrays hold one
-    partial per segment, in the slot of the segment's first partition -- the partials the
-    kernel model gives for a partition size of one segment."""
+def _segment_mark(word):
+    """Segment length that slot 1 of a row of max_logits tells (None: no mark there)."""
+    bits = int(word.view(torch.int32).item()) & 0xFFFFFFFF
+    return (bits & 0xFF) if (bits & 0xFFFFFF00) == 0x7FD3A600 else None
+
+
+@pytest.mark.parametrize("batch", ["many_short", "few_long", "one_partition_each"])
+def test_segment_kernel_partials_lie_a_segment_apart(oracle, batch):
+    """Batches that the split path works in segments of several partitions: the output matches the
+    oracle, and the scratch arrays hold one partial per segment, in the slot of the segment's
+    first partition -- the partials the kernel model gives for a partition size of one segment --
+    and, in slot 1 of max_logits of every row of two or more partitions, the mark by which the
+    reduce kernel learns the segment length."""
     gen = torch.Generator().manual_seed(21)
-    S = 64
-    lens = torch.randint(1, 5000, (S,), generator=gen)
-    lens[5] = 0
-    lens[6] = 4096          # ends exactly on a partition boundary
-    w = W.make_config(4, num_seqs=S, pool_blocks=S * 320, lens=lens.tolist())   # bf16 queries, E5M2 pools, G = 8
+    if batch == "many_short":     # many sequences per compute unit: most sequences are one segment
+        S = 64
+        lens = torch.randint(1, 5000, (S,), generator=gen)
+        lens[5] = 0
+        lens[6] = 4096          # ends exactly on a partition boundary
+    elif batch == "few_long":   # whole segments are the work: one per compute unit
+        S = 5
+        lens = torch.randint(6000, 20000, (S,), generator=gen)
+        lens[1] = 300           # a row of one partition: nothing to mark
+        lens[3] = 0
+    else:                       # no sequence reaches a second partition, though there are slots for two
+        S = 200
+        lens = torch.randint(1, 512, (S,), generator=gen)
+    w = W.make_config(4, num_seqs=S, pool_blocks=int(sum(-(-int(n) // 16) for n in lens)) + 8,
+                      lens=lens.tolist())   # bf16 queries, E5M2 pools, G = 8
     w.sinks = torch.linspace(-1, 3, w.num_heads).to(w.query.dtype)
     from flash_attention_factory_amd import runner
     wd = w.to(_dev())
-    bufs = runner.alloc_buffers(wd)
+    bufs = runner.alloc_buffers(wd, max_num_partitions=2 if batch == "one_partition_each" else None)
     for t in (bufs.exp_sums, bufs.max_logits, bufs.tmp_out):
         t.fill_(float("nan"))
     runner.run_workload(wd, "fp8_reduce", bufs)
@@ -246,23 +264,31 @@ def test_segment_kernel_partials_lie_a_segment_apart(oracle):
     ref = call_oracle(oracle.attention_ref, w)
     live = lens > 0
     torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
-    # which slots were written: 0, m, 2m, ...
     es = bufs.exp_sums.cpu()
+    ml = bufs.max_logits.cpu()
+    P = w.partition_size
+    if batch == "one_partition_each":
+        # one partial per row, in slot 0; slot 1 is nobody's: whatever it holds, nothing reads it
+        assert (~torch.isnan(es[live][:, :, 0])).all() and torch.isnan(es[:, :, 1]).all()
+        return
+    # which slots were written: 0, m, 2m, ...
     longest = int(lens.argmax())
     written = (~torch.isnan(es[longest, 0])).nonzero().flatten().tolist()
     assert written[0] == 0 and len(written) >= 2
     m = written[1]
     assert m >= 2, "this batch is meant to be cut into multi-partition segments"
-    P = w.partition_size
     for s in range(S):
         nseg = -(-int(lens[s]) // (m * P))
         want = [j * m for j in range(nseg)]
         assert (~torch.isnan(es[s, 0])).nonzero().flatten().tolist() == want, s
+        for h in range(w.num_heads):  # the mark: on every row with a second partition, nowhere else
+            mark = _segment_mark(ml[s, h, 1])
+            assert mark == (m if int(lens[s]) > P else None), (s, h, mark)
     NP = bufs.exp_sums.shape[2]
     mes, mml, mtmp = call_oracle(oracle.kernel_partition, w, partition_size=m * P, max_num_partitions=NP)
     for s in range(S):
         for j in range(-(-int(lens[s]) // (m * P))):
-            torch.testing.assert_close(bufs.max_logits[s, :, j * m].cpu(), mml[s, :, j], atol=1e-3, rtol=1e-4)
+            torch.testing.assert_close(ml[s, :, j * m], mml[s, :, j], atol=1e-3, rtol=1e-4)
             torch.testing.assert_close(es[s, :, j * m], mes[s, :, j], atol=1e-3, rtol=2e-3)
             torch.testing.assert_close(bufs.tmp_out[s, :, j * m].cpu(), mtmp[s, :, j], atol=1e-2, rtol=1e-2)
 
