@@ -93,13 +93,14 @@ __device__ __forceinline__ void count_segments(const int (&ctxv)[NQ], const int 
 //
 // Work-groups g and g + cus share a compute unit, and what a compute unit streams is what
 // bounds the launch: the length aims at a share of the mean load of a compute unit
-// (segment_share_of_load), or at the mean load of a work-group where several share one and the
-// whole segments are the work.  Whole segments are all of one length, and where they pile up
-// that length is what the launch waits for; so: with few sequences on shared units, one segment
+// (segment_share_of_load), or, where work-groups share a unit and the whole segments are the
+// work, at the mean load of a work-group (two on a unit) or half of it (three or more).  With one
+// or two work-groups per unit, whole segments -- all of one length -- must not pile up, for that
+// length is then what the launch waits for; so: with at most one sequence per unit, one segment
 // per unit if that fits (phase 0 below); else no more whole segments than work-groups (the
-// length grows until that holds), and, with two work-groups per compute unit, not a count of
-// segments between one per unit and most of the work-groups (some units would hold two and
-// stream twice as long as the others; the length grows until every unit holds one).
+// length grows until that holds), and, with few sequences, not a count of segments between one
+// per unit and most of the work-groups (some units would hold two and stream twice as long as
+// the others; the length grows until every unit holds one).
 template <int NQ>
 __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], const int (&parts)[NQ],
                                                       int total_partitions, int S, int partition_size,
@@ -114,18 +115,22 @@ __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], con
   const float per_unit = __builtin_amdgcn_rcpf((float)units);
   const float seqs_per_cu = fminf((float)live * (float)num_kv_heads * per_unit, 1024.f);
   int share = segment_share_of_load((int)(seqs_per_cu * 1024.f));
-  if (sharing > 1) share = min(share, sharing == 2 ? 512 : 1024 / sharing);
+  // two on a unit: a whole segment is what a work-group gets; three or more (the head-size-64
+  // instances, whose items are short): two segments per work-group, so that one's start overlaps the
+  // other's merge -- measured on ten such batches, 3-8 % faster than one per work-group
+  if (sharing > 1) share = min(share, sharing == 2 ? 512 : 512 / sharing);
   int m = (int)fminf(items * per_unit * ((float)share * (1.0f / 1024.f)) + 0.5f, (float)kSegmentMaxPartitions);
   m = max(m, 1);
   if (m == 1 && items <= (float)groups) return 1;  // a partition per work-group at most: nothing to weigh
-  // Few sequences on shared compute units: first try one segment per unit (the shortest length
-  // that leaves no more segments than units), as long as a segment is then at most 1.25 of a
-  // unit's mean load -- a work-group alone on its unit streams that much faster than its share.
+  if (sharing > 2) return m;
+  // At most one sequence per shared compute unit: first try one segment per unit (the shortest
+  // length that leaves no more segments than units), as long as a segment is then at most 1.25 of
+  // a unit's mean load -- a work-group alone on its unit streams that much faster than its share.
   const long long items_all = (long long)total_partitions * num_kv_heads;
   const bool few = sharing > 1 && 2 * live * num_kv_heads <= units;
   const int aimed = m;
   int phase = 1;  // 0: one segment per unit; 1: no more whole segments than work-groups; 2: not between
-  if (few && items_all > units) {
+  if (sharing > 1 && live * num_kv_heads <= units && items_all > units) {
     phase = 0;
     m = (int)fminf(ceilf(items * per_unit), (float)kSegmentMaxPartitions);
   }
