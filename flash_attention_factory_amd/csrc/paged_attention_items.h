@@ -103,7 +103,7 @@ struct SegmentItems {
   int S, Hk, m, seg_tokens, full_total, total_items, lane;
 
   // Lane holds sequences lane, lane + 64, ...  m, the partitions per segment, follows from the
-  // batch and the number of work-groups (partitions_per_segment), as in the reduce kernel.
+  // batch, the number of work-groups and the compute units they share (partitions_per_segment).
   __device__ __forceinline__ void build(const PagedAttnParams &p, int lane_, int groups) {
     lane = lane_;
     S = p.num_seqs;

@@ -9,13 +9,14 @@
 // of m consecutive partitions of one (sequence, kv head): its wavefronts interleave the
 // segment's chunks, merge their states in LDS (no barrier: the deferred merge of the
 // persistent loop kernel) and write ONE partial into the slot of the segment's first
-// partition.  The other m - 1 slots are neither written nor read: the reduce kernel is told
-// m and visits slots 0, m, 2m, ...
+// partition.  Of the other m - 1 slots only slot 1 of max_logits is written, with m itself
+// (segment_mark): the reduce kernel reads it there and visits slots 0, m, 2m, ...
 //
-// m is chosen on the device from the batch itself -- all wavefronts, and the reduce kernel
-// after them, evaluate partitions_per_segment() on the same context lengths -- so that there
-// are about two segments per resident work-group: a batch of few long sequences is cut
-// finely, in a batch with a thousand (sequence, kv head) pairs most sequences stay whole.
+// m is chosen on the device from the batch itself -- every wavefront evaluates
+// partitions_per_segment() on the same context lengths -- so that a segment is about what a
+// compute unit, or a work-group of it, should stream: a batch of few long sequences gets one
+// segment per unit or per work-group, in a batch with a thousand (sequence, kv head) pairs most
+// sequences stay whole.
 // Segments are dealt to the work-groups longest first in snake order (see below).
 // Built for up to 256 sequences; larger batches use the grid form.
 //
