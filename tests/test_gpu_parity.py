@@ -293,6 +293,64 @@ def test_segment_kernel_partials_lie_a_segment_apart(oracle, batch):
             torch.testing.assert_close(bufs.tmp_out[s, :, j * m].cpu(), mtmp[s, :, j], atol=1e-2, rtol=1e-2)
 
 
+def _segment_batches(name):
+    gen = torch.Generator().manual_seed(33)
+    if name == "one_segment_per_unit":      # three long sequences, two work-groups per compute unit
+        lens = [21000, 9000, 15000]
+        w = W.make_config(2, num_seqs=3, pool_blocks=sum(-(-n // 16) for n in lens) + 4, lens=lens)
+        return w, "reduce"
+    if name == "three_groups_per_unit":     # head size 64: three work-groups share a compute unit
+        w = W.make_test_shaped(batch_size=96, nheads=16, nheads_k=4, d=64, seqlen_k=3000, varlen=True,
+                               has_sinks=True, seed=5)
+        w.context_lens[::7] = torch.randint(1, 3000, (14,), generator=gen).to(torch.int32)
+        return w, "reduce"
+    if name == "longest_segment":           # partitions of 64 tokens: the segment length meets its cap
+        S = 64
+        lens = torch.randint(7000, 8193, (S,), generator=gen).tolist()
+        w = W.make_config(4, num_seqs=S, pool_blocks=S * 512 + 8, lens=lens)
+        w.partition_size = 64
+        return w, "fp8_reduce"
+    S = 256                                  # many_sequences: most of them stay whole
+    lens = torch.randint(1, 2600, (S,), generator=gen)
+    lens[::9] = torch.randint(4000, 9000, (29,), generator=gen)
+    w = W.make_config(4, num_seqs=S, pool_blocks=int(sum(-(-int(n) // 16) for n in lens)) + 8, lens=lens.tolist())
+    return w, "fp8_reduce"
+
+
+@pytest.mark.parametrize("name", ["one_segment_per_unit", "three_groups_per_unit", "longest_segment", "many_sequences"])
+def test_segment_length_regimes(oracle, name):
+    """One batch for each way the split path arrives at its segment length (one segment per compute
+    unit; half a work-group's load where three share a unit; the cap of 64 partitions; a share of a
+    unit's load with many sequences): the output matches the oracle, every row of two or more
+    partitions carries the same mark, and exactly the slots 0, m, 2m, ... of its live partitions
+    hold partials."""
+    w, kernel = _segment_batches(name)
+    from flash_attention_factory_amd import runner
+    wd = w.to(_dev())
+    bufs = runner.alloc_buffers(wd)
+    for t in (bufs.exp_sums, bufs.max_logits, bufs.tmp_out):
+        t.fill_(float("nan"))
+    runner.run_workload(wd, kernel, bufs)
+    torch.cuda.synchronize()
+    _check(bufs.out, w, oracle, f"segment lengths, {name}")
+    es = bufs.exp_sums.cpu()
+    ml = bufs.max_logits.cpu()
+    P = w.partition_size
+    lens = [int(n) for n in w.context_lens.tolist()]
+    marks = {_segment_mark(ml[s, 0, 1]) for s in range(len(lens)) if lens[s] > P}
+    assert len(marks) == 1, marks
+    m = marks.pop() or 1
+    print(f"{name}: {m} partitions per segment", flush=True)
+    if name == "longest_segment":
+        assert m == 64
+    elif name != "three_groups_per_unit":
+        assert m > 1
+    for s, n in enumerate(lens):
+        want = [j * m for j in range(-(-n // (m * P)))]
+        for h in (0, w.num_heads - 1):
+            assert (~torch.isnan(es[s, h])).nonzero().flatten().tolist() == want, (s, h)
+
+
 @pytest.mark.parametrize("batch,heads", [(300, 16), (128, 32)])
 def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
     """From 4096 (sequence, head) pairs on the reduce kernel runs one wavefront per pair;
