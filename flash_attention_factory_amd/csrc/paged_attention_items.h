@@ -110,7 +110,8 @@ struct SegmentItems {
     Hk = p.num_kv_heads;
     const int max_ctx = p.max_blocks_per_seq << p.block_shift;
     const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size, p.max_num_partitions, lane, ctxv, parts);
-    m = partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups, p.compute_units);
+    m = partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups, p.compute_units,
+                                   p.kv_rows_apart != 0);
     seg_tokens = m * p.partition_size;
     int running = 0, tails = 0;
 #pragma unroll

@@ -93,18 +93,19 @@ __device__ __forceinline__ void count_segments(const int (&ctxv)[NQ], const int 
 //
 // Work-groups g and g + cus share a compute unit, and what a compute unit streams is what
 // bounds the launch: the length aims at a share of the mean load of a compute unit
-// (segment_share_of_load), or, where work-groups share a unit and the whole segments are the
-// work, at the mean load of a work-group (two on a unit) or half of it (three or more).  With one
-// or two work-groups per unit, whole segments -- all of one length -- must not pile up, for that
-// length is then what the launch waits for; so: with at most one sequence per unit, one segment
-// per unit if that fits (phase 0 below); else no more whole segments than work-groups (the
-// length grows until that holds), and, with few sequences, not a count of segments between one
-// per unit and most of the work-groups (some units would hold two and stream twice as long as
-// the others; the length grows until every unit holds one).
+// (segment_share_of_load), or, where two work-groups share a unit and the whole segments are the
+// work, at the mean load of a work-group; with token rows that lie apart in the pools, or three
+// work-groups on a unit, at half a work-group's load.  With contiguous rows and one or two work-groups per unit, whole segments
+// -- all of one length -- must not pile up, for that length is then what the launch waits for;
+// so: with at most one sequence per unit, one segment per unit if that fits (phase 0 below);
+// else no more whole segments than work-groups (the length grows until that holds), and, with
+// few sequences, not a count of segments between one per unit and most of the work-groups (some
+// units would hold two and stream twice as long as the others; the length grows until every
+// unit holds one).
 template <int NQ>
 __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], const int (&parts)[NQ],
                                                       int total_partitions, int S, int partition_size,
-                                                      int num_kv_heads, int groups, int cus) {
+                                                      int num_kv_heads, int groups, int cus, bool rows_apart) {
   const int units = max(1, min(groups, cus));  // compute units at work
   const int sharing = groups <= units ? 1 : groups <= 2 * units ? 2 : (groups + units - 1) / units;  // work-groups on each
   int live = 0;
@@ -115,14 +116,21 @@ __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], con
   const float per_unit = __builtin_amdgcn_rcpf((float)units);
   const float seqs_per_cu = fminf((float)live * (float)num_kv_heads * per_unit, 1024.f);
   int share = segment_share_of_load((int)(seqs_per_cu * 1024.f));
-  // two on a unit: a whole segment is what a work-group gets; three or more (the head-size-64
-  // instances, whose items are short): two segments per work-group, so that one's start overlaps the
-  // other's merge -- measured on ten such batches, 3-8 % faster than one per work-group
-  if (sharing > 1) share = min(share, sharing == 2 ? 512 : 512 / sharing);
+  // Work-groups sharing a unit.  Token rows that lie apart in the pools (upstream's layout): two
+  // segments per work-group whatever the batch -- a work-group alone on its unit does not stream
+  // scattered rows at the unit's rate, so both of a unit's work-groups should have work
+  // throughout (measured on 25 such batches: within 1.4 % of the best length on average, where the
+  // rule for contiguous rows is 3-8 % off).  The same where three or more share a unit (the
+  // head-size-64 instances: short items, and no batch of theirs measured more than 8 % off with it,
+  // where a longer segment lost 20 % on one).  Contiguous rows, two on a unit: a whole segment is
+  // what a work-group gets.
+  const bool halves = sharing > 2 || (rows_apart && sharing > 1);
+  if (halves) share = 512 / sharing;
+  else if (sharing == 2) share = min(share, 512);
   int m = (int)fminf(items * per_unit * ((float)share * (1.0f / 1024.f)) + 0.5f, (float)kSegmentMaxPartitions);
   m = max(m, 1);
   if (m == 1 && items <= (float)groups) return 1;  // a partition per work-group at most: nothing to weigh
-  if (sharing > 2) return m;
+  if (halves) return m;
   // At most one sequence per shared compute unit: first try one segment per unit (the shortest
   // length that leaves no more segments than units), as long as a segment is then at most 1.25 of
   // a unit's mean load -- a work-group alone on its unit streams that much faster than its share.

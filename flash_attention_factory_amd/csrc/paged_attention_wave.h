@@ -78,9 +78,12 @@ struct PagedAttnParams {
   // kv_head_bytes describe the pairs -- while query and out rows keep 64 elements.  See
   // WaveAttn::kPairable.
   int32_t pair_heads;
-  // compute units of the GPU: the split path's segment length depends on it
-  // (partitions_per_segment)
+  // what the split path's segment length depends on besides the batch (partitions_per_segment):
+  // the compute units of the GPU, and whether the token rows of a kv head lie apart in the pools
+  // (upstream's layout [blocks, block, kv_heads, d]) or on end (a block's rows of one kv head
+  // contiguous)
   int32_t compute_units;
+  int32_t kv_rows_apart;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI
