@@ -54,9 +54,25 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       // two column tiles in the registers of every wavefront: K and V are loaded once for both
       auto two_tiles = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, PW, TwoTile<KV8>::tiles_per_chunk, KROW>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
-      int resident = 0;
-      FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident));
-      const dim3 grid((unsigned)std::min<int64_t>(resident, items));
+      int resident = 0, cus = 0;
+      FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident, &cus));
+      int64_t groups = std::min<int64_t>(resident, items);
+      // FP8 pools in upstream's layout, head size 128: a token's row of one kv head is a single
+      // 128-byte line, and the rows of its neighbours lie next to it.  A work-group then takes two
+      // adjacent kv heads of a sequence, two wavefronts each, so that both lines are asked for at
+      // about the same time (the FP8 loop configuration on such pools: 60.3 -> 54.2 us, what it
+      // takes on head-major pools).  Half as many items: unless they number twice the resident
+      // work-groups, one work-group per compute unit takes them (1.5 items each would leave half
+      // the work-groups waiting for the other half).  16-bit rows are 256 bytes, and gain nothing.
+      if constexpr (KV8 && HEAD_SIZE == 128) {
+        if (!ext && !r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
+          kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk, false, KROW, 2>;
+          const int64_t pairs = items / 2;
+          groups = pairs >= 2 * (int64_t)resident ? resident : std::min<int64_t>(cus, pairs);
+        }
+      }
+      const dim3 grid((unsigned)groups);
       FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
     } else if (KV8 && HEAD_SIZE == 128 && !ext && !r.pair_heads && r.schedule == FA_SCHEDULE_GRID_LDS) {
       // grid form, K and V staged through LDS: one work-group of eight wavefronts per compute unit

@@ -35,9 +35,11 @@ struct LoopItems {
   // Lane holds sequences lane and lane + 64.  Requested together with the lengths, so that the
   // first K/V loads depend on one round trip to memory, not two: for EVERY sequence the block ids
   // of chunk `wave`, the one this wavefront starts an item with (first_id).
-  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane, int wave, int groups, int chunk_tokens) {
+  // heads_per_item: adjacent kv heads that one work-group takes together (its wavefronts in teams)
+  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane, int wave, int groups, int chunk_tokens,
+                                        int heads_per_item = 1) {
     S = p.num_seqs;
-    Hk = p.num_kv_heads;
+    Hk = p.num_kv_heads / heads_per_item;
     const int max_ctx = p.max_blocks_per_seq << p.block_shift;
     const int col_max = p.max_blocks_per_seq - 1;
     if (lane < S) {
@@ -104,10 +106,11 @@ struct SegmentItems {
 
   // Lane holds sequences lane, lane + 64, ...  m, the partitions per segment, follows from the
   // batch, the number of work-groups and the compute units they share (partitions_per_segment).
-  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane_, int groups) {
+  // heads_per_item: adjacent kv heads that one work-group takes together (its wavefronts in teams)
+  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane_, int groups, int heads_per_item = 1) {
     lane = lane_;
     S = p.num_seqs;
-    Hk = p.num_kv_heads;
+    Hk = p.num_kv_heads / heads_per_item;
     const int max_ctx = p.max_blocks_per_seq << p.block_shift;
     const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size, p.max_num_partitions, lane, ctxv, parts);
     m = partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups, p.compute_units,

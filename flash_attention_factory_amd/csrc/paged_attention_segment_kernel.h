@@ -35,10 +35,11 @@
 namespace fa {
 
 //
-template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false>
+template <int D, typename QT, int KVF, int NWG, int OCC, int TPC, bool EXT = false, int HPW = 1>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 paged_attn_segment_kernel(const PagedAttnParams p) {
-  constexpr int NW = NWG;  // wavefronts that share a segment's chunks and merge
+  constexpr int NW = NWG;       // wavefronts of the work-group
+  constexpr int NT = NW / HPW;  // of which a team of NT shares a segment's chunks of one kv head and merges
   using W = WaveAttn<D, QT, KVF, TPC, SegmentSplit<(KVF != 0)>::stream_loads, EXT>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
@@ -47,12 +48,14 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   constexpr int CT = W::CT;
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
-  constexpr int SL = NR / NW;
-  static_assert(NW > 1 && NR % NW == 0 && SL >= 4 && SL % 4 == 0,
+  constexpr int SL = NR / NT;
+  static_assert(NT > 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 4 && SL % 4 == 0,
                 "each wavefront stores whole 16-byte pieces");
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int team = HPW == 1 ? 0 : wave / NT;   // which of the item's HPW adjacent kv heads
+  const int tw = HPW == 1 ? wave : wave % NT;  // wavefront within the team
   const int G = gridDim.x;
   const int col_max = p.max_blocks_per_seq - 1;
 
@@ -61,9 +64,14 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   // come out even although a work-group only gets a handful of segments.
   using Item = WorkItem;  // c_lo .. c_end: the segment's chunks; ctx: the sequence's length (EXT)
   SegmentItems items;
-  items.build(p, lane, G);
-  // n-th item of this work-group
-  auto item_at = [&](int nth, Item &it) { return items.at(nth, G, (int)blockIdx.x, CT, it); };
+  items.build(p, lane, G, HPW);
+  // n-th item of this work-group; with HPW > 1 an item is HPW adjacent kv heads of one segment, of
+  // which this wavefront's team takes one (kvh is then the team's own head)
+  auto item_at = [&](int nth, Item &it) {
+    const bool there = items.at(nth, G, (int)blockIdx.x, CT, it);
+    if constexpr (HPW > 1) it.kvh = it.kvh * HPW + team;
+    return there;
+  };
 
   // Partial states of two items in flight: the n-th item of this work-group goes to buffer n & 1.
   __shared__ float sm_m[2][NW][16];
@@ -117,23 +125,24 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     // the status word (one lane, a plain vector store) and carry on, so that the grid still drains.
     if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int w0 = team * NT;  // the team's wavefronts: w0 .. w0 + NT - 1
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_m[b][w][i]);
-    float f[NW];
+    for (int u = 0; u < NT; ++u) M = fmaxf(M, sm_m[b][w0 + u][i]);
+    float f[NT];
     float L = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const float mw = sm_m[b][w][i];
-      f[w] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
-      L += f[w] * sm_l[b][w][i];
+    for (int u = 0; u < NT; ++u) {
+      const float mw = sm_m[b][w0 + u][i];
+      f[u] = (mw == -INFINITY) ? 0.f : fast_exp2(mw - M);  // a wavefront without chunks
+      L += f[u] * sm_l[b][w0 + u][i];
     }
     float o[SL];
 #pragma unroll
     for (int e = 0; e < SL; ++e) {
       float a = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) a += f[w] * sm_acc[b][w][wave * SL + e][lane];
+      for (int u = 0; u < NT; ++u) a += f[u] * sm_acc[b][w0 + u][tw * SL + e][lane];
       o[e] = a;
     }
     if (wa.col_valid && wa.keeps_output()) {
@@ -145,9 +154,9 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
         inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key of the segment
       }
       const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
-      const int d0 = wa.out_elem(4 * r * NDT + wave * SL);
+      const int d0 = wa.out_elem(4 * r * NDT + tw * SL);
       W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
-      if ((wa.paired() ? (r & 1) == 0 : r == 0) && wave == 0) {  // one lane per column, see merge_and_store
+      if ((wa.paired() ? (r & 1) == 0 : r == 0) && tw == 0) {  // one lane per column, see merge_and_store
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;
         // the first segment of a row of two or more partitions tells the reduce kernel how long
@@ -161,18 +170,18 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   int n = 0;
   clip(cur);
   // first chunk of the first item
-  bool armed = cur.c_lo + wave < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
+  bool armed = cur.c_lo + tw < cur.c_end;  // loads of this wavefront's first chunk of `cur` in flight
   ItemExt cur_ext = {}, nxt_ext = {};            // extended instances only
   TileScales ts = {}, nts = {}, nxt_ts = {};
   if constexpr (EXT) cur_ext = wa.fetch_item_ext(cur.kvh, p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq);
   if (armed) {
-    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_lo + wave, col_max);
+    const Ids ids = wa.fetch_ids(p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq, cur.c_lo + tw, col_max);
     wa.load_q(cur.seq, cur.kvh);
-    wa.issue_k(R, cur.kvh, cur.c_lo + wave, ids);
-    wa.issue_v(R, cur.kvh, cur.c_lo + wave, ids);
+    wa.issue_k(R, cur.kvh, cur.c_lo + tw, ids);
+    wa.issue_v(R, cur.kvh, cur.c_lo + tw, ids);
     if constexpr (EXT) ts = wa.fetch_scales(ids, cur.kvh, cur_ext);
   }
-  uint32_t sink_raw = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
+  uint32_t sink_raw = wa.load_sink(cur.kvh, tw == 0 && cur.part0 == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
   float prev_out_mul = 1.f;
 
@@ -184,33 +193,33 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       if constexpr (EXT)
         nxt_ext = wa.fetch_item_ext(nxt.kvh, p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq);
     }
-    const bool next_armed = has_next && nxt.c_lo + wave < nxt.c_end;
+    const bool next_armed = has_next && nxt.c_lo + tw < nxt.c_end;
     Ids nxt_ids = {};
     if (next_armed)
-      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_lo + wave, col_max);
+      nxt_ids = wa.fetch_ids(p.block_tables + (int64_t)nxt.seq * p.max_blocks_per_seq, nxt.c_lo + tw, col_max);
 
     wa.reset(sink_raw);
     if constexpr (EXT) wa.set_item(cur_ext, cur.ctx);
     uint32_t next_sink = W::kNoSink;
     if constexpr (EXT) {
       // a segment before the local window arms no wavefront, yet its partial carries the sink
-      if (has_next && !next_armed) next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      if (has_next && !next_armed) next_sink = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
     }
     bool owed = n > 0;
     if (armed) {
       const int32_t *table = p.block_tables + (int64_t)cur.seq * p.max_blocks_per_seq;
-      int ci = cur.c_lo + wave;
-      Ids nids = wa.fetch_ids(table, ci + NW, col_max);
-      if (ci + NW < cur.c_end) {
+      int ci = cur.c_lo + tw;
+      Ids nids = wa.fetch_ids(table, ci + NT, col_max);
+      if (ci + NT < cur.c_end) {
         {  // first chunk of the item, then the merge owed to the previous item
-          const int cn = ci + NW;
+          const int cn = ci + NT;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
-          nids = wa.fetch_ids(table, cn + NW, col_max);
+          nids = wa.fetch_ids(table, cn + NT, col_max);
           ts = nts;
           ci = cn;
         }
@@ -218,15 +227,15 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
           finish(n - 1, prev, prev_out_mul);
           owed = false;
         }
-        while (ci + NW < cur.c_end) {  // steady state: the next chunk belongs to the same item
-          const int cn = ci + NW;
+        while (ci + NT < cur.c_end) {  // steady state: the next chunk belongs to the same item
+          const int cn = ci + NT;
           const auto s = wa.qk(R);
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
           wa.pv(R, pb);
           wa.issue_v(R, cur.kvh, cn, nids);
-          nids = wa.fetch_ids(table, cn + NW, col_max);
+          nids = wa.fetch_ids(table, cn + NT, col_max);
           ts = nts;
           ci = cn;
         }
@@ -235,18 +244,18 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       const auto s = wa.qk(R);
       if (next_armed) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
-        next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-        wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+        next_sink = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
+        wa.issue_k(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
         if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
       }
       const auto pb = wa.template soft<true, EXT>(R, s, ci, cur.tok_end, &ts);
       wa.pv(R, pb);
-      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      if (next_armed) wa.issue_v(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
       wa.load_q(nxt.seq, nxt.kvh);
-      next_sink = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-      wa.issue_k(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-      wa.issue_v(R, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      next_sink = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
+      wa.issue_k(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
+      wa.issue_v(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
       if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
     if (owed) finish(n - 1, prev, prev_out_mul);

@@ -351,6 +351,63 @@ def test_segment_length_regimes(oracle, name):
             assert (~torch.isnan(es[s, h])).nonzero().flatten().tolist() == want, (s, h)
 
 
+@pytest.mark.parametrize("shape", ["few_items", "one_group_per_unit", "all_groups", "gqa"])
+def test_fp8_loop_two_kv_heads_per_work_group(oracle, shape):
+    """FP8 pools in upstream's layout with head size 128: the persistent loop kernel gives a
+    work-group two adjacent kv heads of a sequence, a team of two wavefronts each -- fewer pairs
+    than compute units, one work-group per unit, all resident work-groups, and a grouped-query
+    shape; ragged lengths with empty sequences and sinks."""
+    gen = torch.Generator().manual_seed(91)
+    if shape == "gqa":   # 8 kv heads of 8 query heads each, bf16 queries
+        index, S, hi, fp8_dtype = 4, 40, 3000, torch.float8_e4m3fn
+    else:                # 32 kv heads, one query head each, fp16 queries
+        index, fp8_dtype = 3, torch.float8_e5m2
+        S, hi = {"few_items": (6, 2500), "one_group_per_unit": (32, 1200), "all_groups": (128, 300)}[shape]
+    lens = torch.randint(1, hi, (S,), generator=gen)
+    lens[1] = 0
+    lens[2] = 16
+    w = W.make_config(index, num_seqs=S, pool_blocks=int(sum(-(-int(n) // 16) for n in lens)) + 8, lens=lens.tolist(),
+                      layout=W.TOKEN_MAJOR, fp8_dtype=fp8_dtype)
+    w.sinks = torch.linspace(-2, 2, w.num_heads).to(w.query.dtype)
+    bufs, _ = _run(w, "fp8_loop")
+    out = bufs.out.cpu()
+    assert (out[lens == 0] == 0).all()
+    _check(bufs.out, w, oracle, f"loop kernel, two kv heads per work-group, {shape}")
+
+
+@pytest.mark.parametrize("fp8_dtype", [torch.float8_e5m2, torch.float8_e4m3fn])
+def test_fp8_split_two_kv_heads_per_work_group(oracle, fp8_dtype):
+    """FP8 pools in upstream's layout with head size 128: the segment kernel gives a work-group two
+    adjacent kv heads of a segment, a team of two wavefronts each.  Ragged lengths (empty, one chunk,
+    one partition exactly, many segments), sinks: parity with the oracle, partials in the slots
+    0, m, 2m, ... of every head of a pair, one mark per row of two or more partitions."""
+    gen = torch.Generator().manual_seed(77)
+    S = 40
+    lens = torch.randint(1, 3000, (S,), generator=gen)
+    lens[0], lens[3], lens[4], lens[9], lens[17] = 0, 20, 512, 9000, 6100
+    w = W.make_config(4, num_seqs=S, pool_blocks=int(sum(-(-int(n) // 16) for n in lens)) + 8, lens=lens.tolist(),
+                      layout=W.TOKEN_MAJOR, fp8_dtype=fp8_dtype)
+    w.sinks = torch.linspace(-1, 3, w.num_heads).to(w.query.dtype)
+    from flash_attention_factory_amd import runner
+    wd = w.to(_dev())
+    bufs = runner.alloc_buffers(wd)
+    for t in (bufs.exp_sums, bufs.max_logits, bufs.tmp_out):
+        t.fill_(float("nan"))
+    runner.run_workload(wd, "fp8_reduce", bufs)
+    torch.cuda.synchronize()
+    _check(bufs.out, w, oracle, f"two kv heads per work-group, {fp8_dtype}")
+    es = bufs.exp_sums.cpu()
+    ml = bufs.max_logits.cpu()
+    P = w.partition_size
+    marks = {_segment_mark(ml[s, h, 1]) for s in range(S) for h in range(w.num_heads) if int(lens[s]) > P}
+    assert len(marks) == 1, marks
+    m = marks.pop() or 1
+    for s in range(S):
+        want = [j * m for j in range(-(-int(lens[s]) // (m * P)))]
+        for h in range(w.num_heads):
+            assert (~torch.isnan(es[s, h])).nonzero().flatten().tolist() == want, (s, h)
+
+
 @pytest.mark.parametrize("batch,heads", [(300, 16), (128, 32)])
 def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
     """From 4096 (sequence, head) pairs on the reduce kernel runs one wavefront per pair;
