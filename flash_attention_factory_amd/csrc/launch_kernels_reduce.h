@@ -65,12 +65,15 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
       // 128-byte line, and the rows of its neighbours lie next to it.  A work-group then takes two
       // adjacent kv heads of a segment, two wavefronts each, so that both lines are asked for at
       // about the same time (measured with loads alone: 5.8 -> 6.2-6.4 TB/s, what rows of 256
-      // bytes reach; the serving-mix configuration 300 -> 287 us).  With 16-bit caches, whose rows
+      // bytes reach; the serving-mix configuration 300 -> 282 us).  With 16-bit caches, whose rows
       // are 256 bytes, the same arrangement gained nothing.
+      bool head_teams = false;
       if constexpr (KV8 && HEAD_SIZE == 128) {
-        if (!ext && !r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0)
+        if (!ext && !r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
           kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                              Pipeline<KV8>::tiles_per_chunk, false, 2>;
+          head_teams = true;
+        }
       }
       if (q0 == 0) {
         // Every launch of the call gets the same number of work-groups: the segment length, which
@@ -78,6 +81,9 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
         int resident = 0, cus = 0;
         FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident, &cus));
         p.compute_units = cus;
+        // two teams in a work-group stream like two work-groups: one such work-group per compute
+        // unit (measured on the serving mix: 293 us with two per unit, 282 us with one)
+        if (head_teams) resident = std::min(resident, cus);
         if (ext && r.query_len > per_launch && r.query_len % per_launch <= per_tile) {  // a one-tile launch ends the call
           int other = 0;
           FA_HIP_CHECK(resident_groups(extended, SW * 64, &other));
