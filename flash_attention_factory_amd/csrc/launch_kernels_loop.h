@@ -57,14 +57,15 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       int resident = 0, cus = 0;
       FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident, &cus));
       int64_t groups = std::min<int64_t>(resident, items);
-      // FP8 pools in upstream's layout, head size 128: a token's row of one kv head is a single
-      // 128-byte line, and the rows of its neighbours lie next to it.  A work-group then takes two
-      // adjacent kv heads of a sequence, two wavefronts each, so that both lines are asked for at
-      // about the same time (the FP8 loop configuration on such pools: 60.3 -> 54.2 us, what it
-      // takes on head-major pools).  Half as many items: unless they number twice the resident
-      // work-groups, one work-group per compute unit takes them (1.5 items each would leave half
-      // the work-groups waiting for the other half).  16-bit rows are 256 bytes, and gain nothing.
-      if constexpr (KV8 && HEAD_SIZE == 128) {
+      // Pools in upstream's layout whose token rows are 128 bytes (FP8 with head size 128, 16-bit
+      // with head size 64): a token's row of one kv head is a single line, and the rows of its
+      // neighbours lie next to it.  A work-group then takes two adjacent kv heads of a sequence, two
+      // wavefronts each, so that both lines are asked for at about the same time (the FP8 loop
+      // configuration on such pools: 60.3 -> 54.2 us, what it takes on head-major pools; upstream's
+      // 16-bit perf shape 39.0 -> 35.2 us).  Half as many items: unless they number twice the
+      // resident work-groups, one work-group per compute unit takes them (1.5 items each would
+      // leave half the work-groups waiting for the other half).  Rows of 256 bytes gain nothing.
+      if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
         if (!ext && !r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
           kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
                                                      Pipeline<KV8>::tiles_per_chunk, false, KROW, 2>;

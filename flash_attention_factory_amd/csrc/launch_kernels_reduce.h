@@ -61,14 +61,15 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
       // two column tiles in the registers of every wavefront: K and V are loaded once for both
       auto two_tiles = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, SW, TwoTile<KV8>::tiles_per_chunk, true, true>;
       auto kernel = !ext ? plain : p.query_count > per_tile ? two_tiles : extended;
-      // FP8 pools in upstream's layout, head size 128: a token's row of one kv head is a single
-      // 128-byte line, and the rows of its neighbours lie next to it.  A work-group then takes two
+      // Pools in upstream's layout whose token rows are 128 bytes (FP8 with head size 128, 16-bit
+      // with head size 64): a token's row of one kv head is a single line, and the rows of its
+      // neighbours lie next to it.  A work-group then takes two
       // adjacent kv heads of a segment, two wavefronts each, so that both lines are asked for at
       // about the same time (measured with loads alone: 5.8 -> 6.2-6.4 TB/s, what rows of 256
-      // bytes reach; the serving-mix configuration 300 -> 282 us).  With 16-bit caches, whose rows
-      // are 256 bytes, the same arrangement gained nothing.
+      // bytes reach; the serving-mix configuration 300 -> 282 us, upstream's 16-bit perf shape 44.4 ->
+      // 42.0 us).  With rows of 256 bytes the same arrangement gained nothing.
       bool head_teams = false;
-      if constexpr (KV8 && HEAD_SIZE == 128) {
+      if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
         if (!ext && !r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
           kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
                                              Pipeline<KV8>::tiles_per_chunk, false, 2>;
@@ -76,8 +77,8 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
         }
       }
       if (q0 == 0) {
-        // Every launch of the call gets the same number of work-groups: the segment length, which
-        // the reduce kernel works out again, follows from it.
+        // Every launch of the call gets the same number of work-groups: the segment length follows
+        // from it.
         int resident = 0, cus = 0;
         FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident, &cus));
         p.compute_units = cus;
