@@ -66,12 +66,16 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       // resident work-groups, one work-group per compute unit takes them (1.5 items each would
       // leave half the work-groups waiting for the other half).  Rows of 256 bytes gain nothing.
       if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
-        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0 &&
-            kernel != two_tiles) {
-          kernel = ext ? paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                           Pipeline<KV8>::tiles_per_chunk, true, KROW, 2>
-                       : paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
-                                                           Pipeline<KV8>::tiles_per_chunk, false, KROW, 2>;
+        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
+          if (kernel == two_tiles) {
+            kernel = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, PW, TwoTile<KV8>::tiles_per_chunk, KROW, false, 2>;
+            FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident, &cus));
+          } else {
+            kernel = ext ? paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                             Pipeline<KV8>::tiles_per_chunk, true, KROW, 2>
+                         : paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, PW, PersistentLoop<KV8>::occ,
+                                                             Pipeline<KV8>::tiles_per_chunk, false, KROW, 2>;
+          }
           const int64_t pairs = items / 2;
           groups = pairs >= 2 * (int64_t)resident ? resident : std::min<int64_t>(cus, pairs);
         }

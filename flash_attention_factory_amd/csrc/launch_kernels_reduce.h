@@ -70,12 +70,14 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
       // 42.0 us).  With rows of 256 bytes the same arrangement gained nothing.
       bool head_teams = false;
       if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
-        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0 &&
-            kernel != two_tiles) {
-          kernel = ext ? paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                                   Pipeline<KV8>::tiles_per_chunk, true, 2>
-                       : paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
-                                                   Pipeline<KV8>::tiles_per_chunk, false, 2>;
+        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
+          if (kernel == two_tiles)
+            kernel = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, SW, TwoTile<KV8>::tiles_per_chunk, true, true, 2>;
+          else
+            kernel = ext ? paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk, true, 2>
+                         : paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk, false, 2>;
           head_teams = true;
         }
       }

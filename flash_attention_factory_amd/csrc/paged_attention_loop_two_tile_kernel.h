@@ -38,10 +38,11 @@ namespace fa {
 // PART: the split path.  Items are segments of partitions (SegmentItems), what is stored per item
 // and column is a partial -- max, sum and normalised values in exp_sums / max_logits / tmp_out at
 // the slot of the segment's first partition -- and the reduce kernel follows.
-template <int D, typename QT, int KVF, int NWG, int TPC, bool KROW = true, bool PART = false>
+template <int D, typename QT, int KVF, int NWG, int TPC, bool KROW = true, bool PART = false, int HPW = 1>
 __global__ void __launch_bounds__(NWG * 64) __attribute__((amdgpu_waves_per_eu(1)))
 paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
-  constexpr int NW = NWG;  // wavefronts that share an item's chunks and merge
+  constexpr int NW = NWG;       // wavefronts of the work-group
+  constexpr int NT = NW / HPW;  // of which a team of NT shares the chunks of one kv head of an item and merges
   using W = WaveAttn<D, QT, KVF, TPC, PART ? SegmentSplit<(KVF != 0)>::stream_loads : Pipeline<(KVF != 0)>::stream_loads_loop, true, KROW>;
   using Chunk = typename W::Chunk;
   using Ids = typename W::Ids;
@@ -51,11 +52,13 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   constexpr int CT = W::CT;
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
-  constexpr int SL = NR / NW;
-  static_assert(NW > 1 && NR % NW == 0 && SL >= 2, "merge slices the output across wavefronts");
+  constexpr int SL = NR / NT;
+  static_assert(NT > 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 2, "merge slices the output across wavefronts");
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int team = HPW == 1 ? 0 : wave / NT;   // which of the item's HPW adjacent kv heads
+  const int tw = HPW == 1 ? wave : wave % NT;  // wavefront within the team
   const int G = gridDim.x;
   const int wg = blockIdx.x;
   const int col_max = p.max_blocks_per_seq - 1;
@@ -64,12 +67,14 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   const int r = wa.r, i = wa.i;
   using Item = WorkItem;
   std::conditional_t<PART, SegmentItems, LoopItems<TPC>> items;
-  if constexpr (PART) items.build(p, lane, G);
-  else items.build(p, lane, wave, G, CT);
+  if constexpr (PART) items.build(p, lane, G, HPW);
+  else items.build(p, lane, tw, G, CT, HPW);
   // n-th item of this work-group, read from its first chunk that some query token of the launch
   // sees (local window; the launch's earliest query token decides: the same for both tiles)
   auto item_at = [&](int n, Item &it) __attribute__((always_inline)) -> bool {
     if (!items.at(n, G, wg, CT, it)) return false;
+    // with HPW > 1 an item is HPW adjacent kv heads, of which this wavefront's team takes one
+    if constexpr (HPW > 1) it.kvh = it.kvh * HPW + team;
     it.c_lo = wa.first_visible_chunk(it.ctx, it.c_lo);
     return true;
   };
@@ -109,37 +114,38 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   };
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
   auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool mark, float out_mul) __attribute__((always_inline)) {
+    const int w0 = team * NT;  // the team's wavefronts: w0 .. w0 + NT - 1
     float M = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < NW; ++v) M = fmaxf(M, sm_m[tile][b][v][i]);
-    float f[NW];
+    for (int u = 0; u < NT; ++u) M = fmaxf(M, sm_m[tile][b][w0 + u][i]);
+    float f[NT];
     float L = 0.f;
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
-      const float mv = sm_m[tile][b][v][i];
-      f[v] = (mv == -INFINITY) ? 0.f : fast_exp2(mv - M);  // a wavefront without chunks
-      L += f[v] * sm_l[tile][b][v][i];
+    for (int u = 0; u < NT; ++u) {
+      const float mv = sm_m[tile][b][w0 + u][i];
+      f[u] = (mv == -INFINITY) ? 0.f : fast_exp2(mv - M);  // a wavefront without chunks
+      L += f[u] * sm_l[tile][b][w0 + u][i];
     }
     float o[SL];
 #pragma unroll
     for (int k = 0; k < SL; ++k) {
       float a = 0.f;
 #pragma unroll
-      for (int v = 0; v < NW; ++v) a += f[v] * sm_acc[tile][b][v][wave * SL + k][lane];
+      for (int u = 0; u < NT; ++u) a += f[u] * sm_acc[tile][b][w0 + u][tw * SL + k][lane];
       o[k] = a;
     }
     if (w.col_valid) {
       const int head = kvh * p.group + w.col_g;
-      const int d0 = 4 * r * NDT + wave * SL;
+      const int d0 = 4 * r * NDT + tw * SL;
       const int64_t row = (int64_t)seq * p.query_len + w.col_q;
       const float inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key (of the segment)
       if constexpr (PART) {
         const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part0;
         W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
-        if (r == 0 && wave == 0) {  // one lane per column: the true maximum, and the sum against it
+        if (r == 0 && tw == 0) {  // one lane per column: the true maximum, and the sum against it
           float MT = -INFINITY;
 #pragma unroll
-          for (int v = 0; v < NW; ++v) MT = fmaxf(MT, sm_mt[tile][b][v][i]);
+          for (int u = 0; u < NT; ++u) MT = fmaxf(MT, sm_mt[tile][b][w0 + u][i]);
           p.max_logits[slot] = MT * kLn2;  // natural-log units, as upstream stores them
           p.exp_sums[slot] = MT == -INFINITY ? 0.f : L * fast_exp2(M - MT);
           if (mark) p.max_logits[slot + 1] = segment_mark(items.m);  // for the reduce kernel
@@ -175,8 +181,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, mark, out_mul);
   };
   auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
-  // this wavefront's chunks of an item: c_lo + wave, + NW, ... below c_end
-  auto count_of = [&](const Item &it) __attribute__((always_inline)) { return max(0, (it.c_end - it.c_lo - wave + NW - 1) / NW); };
+  // this wavefront's chunks of an item: c_lo + tw, + NW, ... below c_end
+  auto count_of = [&](const Item &it) __attribute__((always_inline)) { return max(0, (it.c_end - it.c_lo - tw + NT - 1) / NT); };
 
   Chunk R0, R1;
   TileScales ts0 = {}, ts1 = {};  // multipliers of the chunks in R0, R1
@@ -193,21 +199,21 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     Ids ids;
     bool have_ids = false;
     if constexpr (!PART) {
-      if (cur.c_lo == 0) {  // the ids requested with the lengths are those of chunk `wave`
+      if (cur.c_lo == 0) {  // the ids requested with the lengths are those of chunk `tw`
 #pragma unroll
         for (int t = 0; t < TPC; ++t) ids.v[t] = min((uint32_t)items.first_id(t, cur.seq), (uint32_t)p.max_block_id);
         have_ids = true;
       }
     }
-    if (!have_ids) ids = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave, col_max);
-    ids1 = wa.fetch_ids(table_of(cur.seq), cur.c_lo + wave + NW, col_max);
+    if (!have_ids) ids = wa.fetch_ids(table_of(cur.seq), cur.c_lo + tw, col_max);
+    ids1 = wa.fetch_ids(table_of(cur.seq), cur.c_lo + tw + NT, col_max);
     wa.load_q(cur.seq, cur.kvh);
     wb.load_q(cur.seq, cur.kvh);
-    wa.issue_k(R0, cur.kvh, cur.c_lo + wave, ids);
-    wa.issue_v(R0, cur.kvh, cur.c_lo + wave, ids);
+    wa.issue_k(R0, cur.kvh, cur.c_lo + tw, ids);
+    wa.issue_v(R0, cur.kvh, cur.c_lo + tw, ids);
     ts0 = wa.fetch_scales(ids, cur.kvh, cur_a);
   }
-  uint32_t sink_a = wa.load_sink(cur.kvh, wave == 0 && cur.part0 == 0), sink_b = wb.load_sink(cur.kvh, wave == 0 && cur.part0 == 0);
+  uint32_t sink_a = wa.load_sink(cur.kvh, tw == 0 && cur.part0 == 0), sink_b = wb.load_sink(cur.kvh, tw == 0 && cur.part0 == 0);
   Item prev = cur;  // the item whose merge is still owed (from the second item on)
   float prev_out_mul = 1.f;
 
@@ -223,8 +229,8 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     const bool next_armed = next_m > 0;
     Ids nxt_ids = {}, nxt_ids1 = {};
     if (next_armed) {
-      nxt_ids = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + wave, col_max);
-      nxt_ids1 = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + wave + NW, col_max);
+      nxt_ids = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + tw, col_max);
+      nxt_ids1 = wa.fetch_ids(table_of(nxt.seq), nxt.c_lo + tw + NT, col_max);
     }
     wa.reset(sink_a);
     wb.reset(sink_b);
@@ -232,33 +238,33 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     wb.set_item(cur_b, cur.ctx);
     uint32_t next_a = W::kNoSink, next_b = W::kNoSink;
     if (has_next && !next_armed) {  // the sink goes with the item whether or not wavefront 0 has a chunk of it
-      next_a = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-      next_b = wb.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      next_a = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
+      next_b = wb.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
     }
     // What the next item needs beyond K and V, once the last scores of this one are out.
     auto request_next_item = [&]() __attribute__((always_inline)) {
       wa.load_q(nxt.seq, nxt.kvh);
       wb.load_q(nxt.seq, nxt.kvh);
-      next_a = wa.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
-      next_b = wb.load_sink(nxt.kvh, wave == 0 && nxt.part0 == 0);
+      next_a = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
+      next_b = wb.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
     };
     TileScales nts = {};
     bool owed = n > 0;  // finish(n - 1) still to do
     if (m > 0) {
       const int32_t *table = table_of(cur.seq);
-      const int c0 = cur.c_lo + wave;  // chunk j of the wavefront is chunk c0 + j * NW of the item
+      const int c0 = cur.c_lo + tw;  // chunk j of the wavefront is chunk c0 + j * NT of the item
       Scores sa, sb;
       Ids ids_a = {}, ids_b = {};  // ids of the chunks R0 and R1 take next
       int j = 0;
       if (m >= 4) {
         // The second chunk: K now; its V loads go out between the MFMAs of the first chunk's scores.
         int64_t vp0[TPC], vp1[TPC];  // where the V loads that R0 / R1 still wait for read from
-        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
+        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NT, ids1);
 #pragma unroll
-        for (int t = 0; t < TPC; ++t) vp1[t] = wa.v_tile_at(cur.kvh, c0 + NW, t, ids1);
+        for (int t = 0; t < TPC; ++t) vp1[t] = wa.v_tile_at(cur.kvh, c0 + NT, t, ids1);
         ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
-        ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
-        ids_b = wa.fetch_ids(table, c0 + 3 * NW, col_max);
+        ids_a = wa.fetch_ids(table, c0 + 2 * NT, col_max);
+        ids_b = wa.fetch_ids(table, c0 + 3 * NT, col_max);
         // One chunk: X holds chunk cx; the chunk two further on takes X over.  A wavefront that has
         // to wait at a load (the memory pipeline is full most of the time) computes nothing
         // meanwhile and there is no second wavefront on its SIMD, so the loads go out one at a
@@ -278,11 +284,11 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           int64_t kp[TPC];
 #pragma unroll
           for (int t = 0; t < TPC; ++t) {
-            kp[t] = wa.k_tile_at(cur.kvh, cx + 2 * NW, t, ids);
-            vpx[t] = wa.v_tile_at(cur.kvh, cx + 2 * NW, t, ids);
+            kp[t] = wa.k_tile_at(cur.kvh, cx + 2 * NT, t, ids);
+            vpx[t] = wa.v_tile_at(cur.kvh, cx + 2 * NT, t, ids);
           }
           nts = wa.fetch_scales(ids, cur.kvh, cur_a);
-          ids = wa.fetch_ids(table, cx + 4 * NW, col_max);
+          ids = wa.fetch_ids(table, cx + 4 * NT, col_max);
           auto k_loads = [&](int part) __attribute__((always_inline)) {  // quarter `part` of the NK loads
 #pragma unroll
             for (int k = part * NK / 4; k < (part + 1) * NK / 4; ++k) {
@@ -308,46 +314,46 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
         __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
         // steady: chunk j in R0 and j+1 in R1 are computed, chunks j+2 and j+3 requested
         while (j + 3 < m) {
-          steady(R0, ts0, vp0, R1, vp1, c0 + j * NW, ids_a);
+          steady(R0, ts0, vp0, R1, vp1, c0 + j * NT, ids_a);
           if (owed) {  // a chunk into the item, the next requests on their way: the merge owed to the item before
             finish(n - 1, prev, prev_out_mul);
             owed = false;
           }
-          steady(R1, ts1, vp1, R0, vp0, c0 + (j + 1) * NW, ids_b);
+          steady(R1, ts1, vp1, R0, vp0, c0 + (j + 1) * NT, ids_b);
           j += 2;
         }
         // the V loads R1 still waits for
 #pragma unroll
         for (int v = 0; v < 4 * TPC; ++v) wa.load_v_one(R1, v / 4, v % 4, vp1[v / 4]);
       } else if (m >= 2) {
-        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NW, ids1);
-        wa.issue_v(R1, cur.kvh, c0 + NW, ids1);
+        if (!k1_ready) wa.issue_k(R1, cur.kvh, c0 + NT, ids1);
+        wa.issue_v(R1, cur.kvh, c0 + NT, ids1);
         ts1 = wa.fetch_scales(ids1, cur.kvh, cur_a);
-        if (m == 3) ids_a = wa.fetch_ids(table, c0 + 2 * NW, col_max);
+        if (m == 3) ids_a = wa.fetch_ids(table, c0 + 2 * NT, col_max);
       }
       // The one to three chunks that end the item: j in R0, j+1 in R1, j+2 on its way into R0 or
       // requested now.  The last of these steps that uses R0 requests the next item's first chunk,
       // the step that uses R1 the K half of its second.
       k1_ready = false;
       const int rem = m - j;
-      const int ca = c0 + j * NW;
+      const int ca = c0 + j * NT;
       {
         W::qk_two(wa, wb, R0, sa, sb);
         if (rem == 3) {
-          wa.issue_k(R0, cur.kvh, ca + 2 * NW, ids_a);
+          wa.issue_k(R0, cur.kvh, ca + 2 * NT, ids_a);
           nts = wa.fetch_scales(ids_a, cur.kvh, cur_a);
         } else if (next_armed) {
           if (rem == 1) request_next_item();
-          wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+          wa.issue_k(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
         const auto pa = wa.template soft<true, true, true>(R0, sa, ca, cur.tok_end, &ts0);
         const auto pb = wb.template soft<true, true, true>(R0, sb, ca, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
         if (rem == 3) {
-          wa.issue_v(R0, cur.kvh, ca + 2 * NW, ids_a);
+          wa.issue_v(R0, cur.kvh, ca + 2 * NT, ids_a);
         } else if (next_armed) {
-          wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+          wa.issue_v(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
         }
         ts0 = nts;
       }
@@ -355,31 +361,31 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
         W::qk_two(wa, wb, R1, sa, sb);
         if (rem == 2 && next_armed) request_next_item();
         if (next_m >= 2) {
-          wa.issue_k(R1, nxt.kvh, nxt.c_lo + wave + NW, nxt_ids1);
+          wa.issue_k(R1, nxt.kvh, nxt.c_lo + tw + NT, nxt_ids1);
           k1_ready = true;
         }
-        const auto pa = wa.template soft<true, true, true>(R1, sa, ca + NW, cur.tok_end, &ts1);
-        const auto pb = wb.template soft<true, true, true>(R1, sb, ca + NW, cur.tok_end, &ts1);
+        const auto pa = wa.template soft<true, true, true>(R1, sa, ca + NT, cur.tok_end, &ts1);
+        const auto pb = wb.template soft<true, true, true>(R1, sb, ca + NT, cur.tok_end, &ts1);
         W::pv_two(wa, wb, R1, pa, pb);
       }
       if (rem == 3) {
         W::qk_two(wa, wb, R0, sa, sb);
         if (next_armed) {
           request_next_item();
-          wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+          wa.issue_k(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
           nts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
         }
-        const auto pa = wa.template soft<true, true, true>(R0, sa, ca + 2 * NW, cur.tok_end, &ts0);
-        const auto pb = wb.template soft<true, true, true>(R0, sb, ca + 2 * NW, cur.tok_end, &ts0);
+        const auto pa = wa.template soft<true, true, true>(R0, sa, ca + 2 * NT, cur.tok_end, &ts0);
+        const auto pb = wb.template soft<true, true, true>(R0, sb, ca + 2 * NT, cur.tok_end, &ts0);
         W::pv_two(wa, wb, R0, pa, pb);
-        if (next_armed) wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+        if (next_armed) wa.issue_v(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
         ts0 = nts;
       }
     } else if (next_armed) {  // nothing to do in `cur`, but the next item starts here
       k1_ready = false;
       request_next_item();
-      wa.issue_k(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
-      wa.issue_v(R0, nxt.kvh, nxt.c_lo + wave, nxt_ids);
+      wa.issue_k(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
+      wa.issue_v(R0, nxt.kvh, nxt.c_lo + tw, nxt_ids);
       ts0 = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_a);
     }
     if (owed) finish(n - 1, prev, prev_out_mul);
