@@ -66,7 +66,10 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       // resident work-groups, one work-group per compute unit takes them (1.5 items each would
       // leave half the work-groups waiting for the other half).  Rows of 256 bytes gain nothing.
       if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
-        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
+        // (with fewer pairs than compute units the GPU is short of work-groups, and halving their
+        // number would cost more than the rows gain)
+        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0 &&
+            items / 2 >= cus) {
           if (kernel == two_tiles) {
             kernel = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, PW, TwoTile<KV8>::tiles_per_chunk, KROW, false, 2>;
             FA_HIP_CHECK(resident_groups(kernel, PW * 64, &resident, &cus));

@@ -68,9 +68,15 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
       // about the same time (measured with loads alone: 5.8 -> 6.2-6.4 TB/s, what rows of 256
       // bytes reach; the serving-mix configuration 300 -> 282 us, upstream's 16-bit perf shape 44.4 ->
       // 42.0 us).  With rows of 256 bytes the same arrangement gained nothing.
+      // Not for batches that cannot give every compute unit a pair even at one partition per
+      // segment (a single sequence of 32 partitions and 8 kv heads: 19.2 us against 15.9 us).
       bool head_teams = false;
       if constexpr (HEAD_SIZE * (KV8 ? 1 : 2) == 128) {  // token rows of 128 bytes
-        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0) {
+        int units = 0, unused = 0;
+        FA_HIP_CHECK(resident_groups(kernel, SW * 64, &unused, &units));
+        const int64_t most_pairs = (int64_t)shape.num_seqs * shape.max_num_partitions * (p.num_kv_heads / 2);
+        if (!r.pair_heads && p.kv_rows_apart && shape.kv_head_stride == shape.head_size && p.num_kv_heads % 2 == 0 &&
+            most_pairs >= units) {
           if (kernel == two_tiles)
             kernel = paged_attn_loop_two_tile_kernel<HEAD_SIZE, QT, KVF, SW, TwoTile<KV8>::tiles_per_chunk, true, true, 2>;
           else
