@@ -296,6 +296,38 @@ def test_two_tile_kernels_at_the_edges_of_their_item_lists(oracle, fp8, qdtype, 
         assert_close_to_reference(got[live], ref[live], f"{kernel} fp8={fp8} block_scales={block_scales}")
 
 
+@pytest.mark.parametrize("cache", ["e5m2", "fp16_head_size_64"])
+def test_two_tile_kernels_with_two_kv_heads_per_work_group(oracle, cache):
+    """Pools in upstream's layout with token rows of 128 bytes and enough pairs of kv heads to give
+    every compute unit one: the two-tile kernels of both paths then hand a work-group two adjacent
+    kv heads, two wavefronts each.  280 pairs, two column tiles (2 heads x 16 tokens), lengths from
+    empty to three partitions, a window, ALiBi and sinks."""
+    fp8 = cache == "e5m2"
+    D = 128 if fp8 else 64
+    S, QL, H, Hk = 140, 16, 8, 4
+    qdtype = torch.bfloat16 if fp8 else torch.float16
+    w = W.make_test_shaped(batch_size=S, nheads=H, nheads_k=Hk, d=D, seqlen_k=700, varlen=False, has_sinks=True,
+                           fp8=fp8, block_size=16, seed=31, dtype=qdtype)
+    g = torch.Generator().manual_seed(19)
+    w.context_lens = torch.randint(1, 701, (S,), generator=g).to(torch.int32)
+    w.context_lens[3], w.context_lens[4], w.context_lens[11] = 0, 7, 700
+    w.sinks = torch.linspace(-2, 2, H).to(qdtype)
+    query4 = torch.randn(S, QL, H, D, generator=g).to(qdtype)
+    alibi = torch.linspace(0.001, 0.02, H)
+    ref = oracle.attention_ref(query4, w.key_cache, w.value_cache, w.block_tables, w.context_lens, scale=w.scale,
+                               block_size=w.block_size, kv_strides=w.kv_strides(), num_kv_heads=w.num_kv_heads,
+                               sinks=w.sinks, fp8_scale=w.fp8_scale, want_f32=True, alibi_slopes=alibi,
+                               window_left=300)[1]
+    wd = w.to(_dev())
+    live = w.context_lens > 0
+    for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+        got = _call_multi(wd, query4.to(_dev()), kernel, alibi_slopes=alibi.to(_dev()), apply_alibi=True,
+                          window_left=300).float().cpu()
+        assert torch.isfinite(got).all(), kernel
+        assert (got[~live] == 0).all(), kernel
+        assert_close_to_reference(got[live], ref[live], f"{kernel} {cache}")
+
+
 @pytest.mark.parametrize("index,QL", [(4, 4), (1, 32), (2, 8)])
 def test_full_size_query_blocks_with_modifiers(oracle, index, QL):
     """The measured configurations at full size with a query block of two column tiles (G x QL =
