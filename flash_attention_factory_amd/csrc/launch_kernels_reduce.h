@@ -187,8 +187,8 @@ inline bool segment_form_fits(const fa_paged_attention_shape &shape) {
 }
 
 // A batch of more sequences than the segment kernel lists is cut into equal sub-batches, each
-// with its own segment and reduce launch (the two agree on the segment length through the
-// sub-batch's context lengths): measured on a 512-sequence serving mix, 56 % of peak in the
+// with its own segment and reduce launch (every attention launch chooses its segment length and
+// marks its rows with it): measured on a 512-sequence serving mix, 56 % of peak in the
 // grid form against 71 % for 256 sequences in the segment form.
 template <int HEAD_SIZE, typename QT, int KVF>
 inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *key_cache,
