@@ -58,6 +58,14 @@ struct LoopItems {
     // (lengths stay below 2^24, the launcher sees to that).  Lanes without a sequence: -1.
     key0 = len0 < 0 ? -1 : (len0 << 7) | (127 - lane);
     key1 = len1 < 0 ? -1 : (len1 << 7) | (63 - lane);
+    // No more items than work-groups: nobody takes a second one, so any order deals them as well
+    // as the sorted one -- skip the ranking (a third of a microsecond of a launch that then lasts
+    // a handful).
+    if (S * Hk <= groups) {
+      rank0 = lane;
+      rank1 = lane + 64;
+      return;
+    }
     // eight sequences per trip; lanes past the batch hold -1 and count for nothing
     for (int u0 = 0; u0 < min(S, 64); u0 += 8) {
 #pragma unroll
