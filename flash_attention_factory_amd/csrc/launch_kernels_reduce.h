@@ -41,7 +41,7 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float attention_us = 0.f;
   const bool segment_form = SegmentSplit<KV8>::use && r.schedule == FA_SCHEDULE_AUTO && shape.num_seqs <= kSegmentMaxSeqs &&
-                            shape.num_pool_blocks > 0 &&
+                            shape.num_pool_blocks > 0 && r.partition_size < kSegmentMaxContext &&
                             (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
   // columns, or in the segment form two tiles of 16 held by every wavefront.
@@ -202,6 +202,7 @@ inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *
   // dimension holds
   constexpr int kGridMaxSeqs = 65535;
   const bool segment_pieces = r.schedule == FA_SCHEDULE_AUTO && segment_form_fits<(KVF != kKv16)>(shape) &&
+                              r.partition_size < kSegmentMaxContext &&
                               shape.num_seqs > kSegmentMaxSeqs;
   const int most = segment_pieces ? kSegmentMaxSeqs : kGridMaxSeqs;
   if (shape.num_seqs > most) {
