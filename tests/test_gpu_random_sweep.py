@@ -61,13 +61,71 @@ def _draw_case(rng):
                 sinks=rng.random() < 0.5, feats=feats, fp8_scale=fp8_scale, seed=rng.randint(0, 1 << 30))
 
 
+def _draw_large_case(rng):
+    """Batches of more (sequence, kv head) items than the GPU has compute units, short contexts:
+    where the kernels rank more than 64 sequences, deal several items to a work-group, put two or
+    three work-groups on a unit and give a work-group two kv heads (pools in upstream's layout with
+    128-byte token rows)."""
+    D, cache = rng.choice([(128, "e5m2"), (128, "e4m3"), (64, "16"), (128, "16"), (64, "e5m2")])
+    Hk = rng.choice([8, 16, 32])
+    G = rng.choice([1, 1, 2, 4, 5])
+    S = rng.choice([rng.randint(17, 64), rng.randint(65, 128), rng.randint(129, 256), rng.randint(257, 300)])
+    psize = rng.choice([256, 512])
+    budget = (24 << 20) // (Hk * D)  # tokens in the pools: the oracle and the random draw stay quick
+    top = min(rng.choice([90, 400, 1500]), max(30, 2 * budget // S))
+    lens = []
+    for _ in range(S):
+        kind = rng.random()
+        if kind < 0.05:
+            lens.append(0)
+        elif kind < 0.15:
+            lens.append(rng.randint(1, 20))
+        elif kind < 0.25:
+            lens.append(max(1, min(top, psize * rng.randint(1, 3) + rng.choice([-1, 0, 1]))))
+        else:
+            lens.append(rng.randint(1, top))
+    if rng.random() < 0.3:   # one sequence far longer than the others
+        lens[rng.randrange(S)] = rng.randint(budget // 4, budget // 2)
+    feats = {}
+    if rng.random() < 0.4:
+        if rng.random() < 0.5:
+            feats["window_left"] = rng.choice([17, 200, 1000])
+        if rng.random() < 0.4:
+            feats["alibi"] = True
+        if rng.random() < 0.5 and S * G * Hk <= 8192:
+            feats["query_len"] = rng.choice([2, 3])
+        if cache != "16" and rng.random() < 0.4:
+            feats["scales"] = rng.choice(["head", "block"])
+    return dict(D=D, Hk=Hk, G=G, B=rng.choice([16, 16, 64]), S=S, cache=cache,
+                qdtype=rng.choice([torch.float16, torch.bfloat16]),
+                layout=rng.choice([W.TOKEN_MAJOR, W.TOKEN_MAJOR, W.HEAD_MAJOR]), psize=psize, lens=lens,
+                sinks=rng.random() < 0.5, feats=feats, fp8_scale=1.0, seed=rng.randint(0, 1 << 30), compact=True)
+
+
+def _compact_pools(w, c, fp8_dtype):
+    """Pools of just the blocks the lengths need (make_test_shaped sizes them for the longest
+    length times the batch), dealt to the sequences in random order."""
+    gen = torch.Generator().manual_seed(c["seed"] + 2)
+    B, Hk, D = c["B"], c["Hk"], c["D"]
+    NB = sum(-(-n // B) for n in c["lens"]) + 3
+    w.block_tables = W._deal_block_tables(c["lens"], B, torch.randperm(NB, generator=gen).to(torch.int32))
+    shape = (NB, B, Hk, D) if c["layout"] == W.TOKEN_MAJOR else (NB, Hk, B, D)
+    w.key_cache = W._randn16(shape, gen, c["qdtype"])
+    w.value_cache = W._randn16(shape, gen, c["qdtype"])
+    if c["cache"] != "16":
+        w.key_cache, w.value_cache = w.key_cache.to(fp8_dtype), w.value_cache.to(fp8_dtype)
+
+
 def _run_case(oracle, c):
     dev = _dev()
     fp8 = c["cache"] != "16"
+    fp8_dtype = torch.float8_e4m3fn if c["cache"] == "e4m3" else torch.float8_e5m2
     w = W.make_test_shaped(batch_size=c["S"], nheads=c["Hk"] * c["G"], nheads_k=c["Hk"], d=c["D"],
-                           seqlen_k=max(c["lens"]), varlen=False, has_sinks=c["sinks"], fp8=fp8, block_size=c["B"],
-                           seed=c["seed"], dtype=c["qdtype"], layout=c["layout"],
-                           fp8_dtype=torch.float8_e4m3fn if c["cache"] == "e4m3" else torch.float8_e5m2)
+                           seqlen_k=c["B"] if c.get("compact") else max(c["lens"]), varlen=False, has_sinks=c["sinks"],
+                           fp8=fp8, block_size=c["B"], seed=c["seed"], dtype=c["qdtype"], layout=c["layout"],
+                           fp8_dtype=fp8_dtype)
+    if c.get("compact"):
+        _compact_pools(w, c, fp8_dtype)
     w.context_lens = torch.tensor(c["lens"], dtype=torch.int32)
     w.partition_size = c["psize"]
     w.fp8_scale = c["fp8_scale"]
@@ -129,4 +187,13 @@ def test_random_cases(oracle, seed):
     for _ in range(CASES_PER_SEED):
         c = _draw_case(rng)
         print(c, flush=True)
+        _run_case(oracle, c)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_large_batches(oracle, seed):
+    rng = random.Random(5000 + seed)
+    for _ in range(5):
+        c = _draw_large_case(rng)
+        print({k: (v if k != "lens" else (len(v), max(v))) for k, v in c.items()}, flush=True)
         _run_case(oracle, c)
