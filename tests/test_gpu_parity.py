@@ -423,21 +423,23 @@ def test_reduce_kernel_one_wavefront_form(oracle, batch, heads):
     _check(bufs.out, w, oracle, f"reduce 1-wave form, {batch} sequences x {heads} heads")
 
 
+@pytest.mark.parametrize("layout", [W.HEAD_MAJOR, W.TOKEN_MAJOR])
 @pytest.mark.parametrize("index", [1, 2, 3, 4])
-def test_full_size_configs(oracle, index):
-    """The measured configurations at their full sizes.  The pools are drawn on the GPU
+def test_full_size_configs(oracle, index, layout):
+    """The measured configurations at their full sizes, in both pool layouts (in upstream's, the
+    FP8 configurations run the instances that give a work-group two kv heads).  The pools are drawn on the GPU
     (a gigabyte of normals takes the host a minute) and copied back for the oracle, so
     both sides see the same bytes.  Also checked at full size: loop == split + reduce,
     and invariance under a permutation of the pool's blocks together with the tables."""
     from flash_attention_factory_amd import runner
     dev = _dev()
-    wd = W.make_config(index, device=dev, pools_on_device=True)
+    wd = W.make_config(index, device=dev, pools_on_device=True, layout=layout)
     w = wd.to("cpu")
     kernel = W.CONFIG_KERNEL[index]
     bufs = runner.alloc_buffers(wd)
     runner.run_workload(wd, kernel, bufs)
     torch.cuda.synchronize()
-    _check(bufs.out, w, oracle, f"full {w.name}")
+    _check(bufs.out, w, oracle, f"full {w.name}, {layout}")
     other = {"loop": "reduce", "reduce": "loop", "fp8_loop": "fp8_reduce", "fp8_reduce": "fp8_loop"}[kernel]
     bufs2 = runner.alloc_buffers(wd)
     runner.run_workload(wd, other, bufs2)
