@@ -293,6 +293,7 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.kv_token_bytes = s.kv_token_stride * r.kv_elem_bytes;
   p.kv_head_bytes = s.kv_head_stride * r.kv_elem_bytes;
   p.compute_units = 0;  // the split path's launcher fills it in
+  p.final_out = nullptr;  // (and this, in the segment form)
   p.kv_rows_apart = s.kv_token_stride != s.head_size;
   p.pair_heads = 0;
   if (r.pair_heads) {  // the kernel sees pairs of kv heads: half as many, twice the group, rows of two heads

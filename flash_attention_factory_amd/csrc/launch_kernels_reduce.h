@@ -46,6 +46,7 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
   // columns, or in the segment form two tiles of 16 held by every wavefront.
   // Every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
+  if (segment_form) p.final_out = out;  // rows of one partial are stored as results (PagedAttnParams::final_out)
   const int per_tile = p.query_count;
   const int per_launch = (segment_form && r.query_len > per_tile) ? 2 * per_tile : per_tile;
   for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {

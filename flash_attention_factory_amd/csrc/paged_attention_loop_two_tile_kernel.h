@@ -113,7 +113,9 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     if (lane == 0) __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
-  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool mark, float out_mul) __attribute__((always_inline)) {
+  // whole: the item is the row's only partial, which goes to the call's `out` as its result
+  // (PagedAttnParams::final_out)
+  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool mark, bool whole, float out_mul) __attribute__((always_inline)) {
     const int w0 = team * NT;  // the team's wavefronts: w0 .. w0 + NT - 1
     float M = -INFINITY;
 #pragma unroll
@@ -141,7 +143,10 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
       const float inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key (of the segment)
       if constexpr (PART) {
         const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + part0;
-        W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
+        if (whole)
+          W::template store_q<SL>(reinterpret_cast<char *>(p.final_out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
+        else
+          W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * D + d0, o, inv);
         if (r == 0 && tw == 0) {  // one lane per column: the true maximum, and the sum against it
           float MT = -INFINITY;
 #pragma unroll
@@ -177,8 +182,10 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     // a row of two or more partitions: its first segment leaves the segment length (segment_mark)
     bool mark = false;
     if constexpr (PART) mark = it.part0 == 0 && items.m > 1 && it.ctx > p.partition_size && p.max_num_partitions > 1;
-    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, mark, out_mul);
-    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, mark, out_mul);
+    bool whole = false;
+    if constexpr (PART) whole = p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx;
+    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, mark, whole, out_mul);
+    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, mark, whole, out_mul);
   };
   auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
   // this wavefront's chunks of an item: c_lo + tw, + NW, ... below c_end

@@ -5,6 +5,8 @@
 //   M = max_p m_p; w_p = l_p * exp(m_p - M)            (rescale_exp_sums :736-764)
 //   out = sum_p (w_p / sum_q w_q) * tmp_out[p, :]      (compute_out :771-864, collect_out :868-934)
 // Only the ceil(context_len / partition_size) live partitions are read (:679,716).
+// After the segment attention kernels a row of a single partial is left alone: the attention
+// kernel has stored it into `out` already.
 //
 // One work-group of one or four wavefronts per (sequence, head).  The kernel is a chain
 // of dependent memory round trips, so it is built to have as few of them as possible:
@@ -77,6 +79,12 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   if constexpr (SEGMENTS) {
     if (np > 1) stride = __builtin_amdgcn_readfirstlane(segment_length_of(slot1));
     np = (np + stride - 1) / stride;  // from here on: the number of partials
+    // one partial: the segment kernel has stored it into `out` as the row's result
+    // (PagedAttnParams::final_out), and its tmp_out row holds nothing
+    if (np == 1) return;
+#ifdef FA_X_DIRECT
+    if (np == 1) return;
+#endif
   }
   const float *ml = p.max_logits + base;
   const float *es = p.exp_sums + base;

@@ -11,6 +11,10 @@
 // persistent loop kernel) and write ONE partial into the slot of the segment's first
 // partition.  Of the other m - 1 slots only slot 1 of max_logits is written, with m itself
 // (segment_mark): the reduce kernel reads it there and visits slots 0, m, 2m, ...
+// A sequence that fits one segment has one partial, which is its result: that one is rounded to
+// the query type and stored into the call's `out` (PagedAttnParams::final_out), its scalars into
+// exp_sums and max_logits as ever, and the reduce kernel leaves the row alone -- in a batch of
+// many sequences that is most rows, and spares them the trip through tmp_out.
 //
 // m is chosen on the device from the batch itself -- every wavefront evaluates
 // partitions_per_segment() on the same context lengths -- so that a segment is about what a
@@ -155,7 +159,18 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       }
       const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
       const int d0 = wa.out_elem(4 * r * NDT + tw * SL);
-      W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
+#ifdef FA_X_DIRECT
+      if (it.part0 == 0 && it.tok_end >= it.ctx)  // timing only: the row's only partial, as 16-bit values
+        W::template store_q<SL>(reinterpret_cast<char *>(p.out) + (slot * wa.out_row_elems()) * 4 + d0 * 2, o, inv);
+      else
+#endif
+      // the row's only partial is its result (PagedAttnParams::final_out); it.ctx is the length as
+      // far as the scratch arrays hold it
+      if (p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx)
+        W::template store_q<SL>(
+            reinterpret_cast<char *>(p.final_out) + ((row * p.num_heads + head) * wa.out_row_elems() + d0) * 2, o, inv);
+      else
+        W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
       if ((wa.paired() ? (r & 1) == 0 : r == 0) && tw == 0) {  // one lane per column, see merge_and_store
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;

@@ -84,6 +84,11 @@ struct PagedAttnParams {
   // contiguous)
   int32_t compute_units;
   int32_t kv_rows_apart;
+  // Split path, segment form: the call's `out`.  A row whose context fits one segment has one
+  // partial, which is its result: the attention kernel rounds it to the query type and stores it
+  // here, not into tmp_out (exp_sums and max_logits still get the partial's scalars), and the reduce
+  // kernel leaves such rows alone.  NULL: every partial goes to tmp_out.
+  void *final_out;
 };
 
 constexpr int kMaskAlibi = 1, kMaskSoftcap = 2, kMaskWindow = 4;  // = fa_mask of the C ABI

@@ -183,7 +183,9 @@ int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_ca
  * (sequence, kv head) pairs one partial covers several consecutive partitions and sits in
  * the slot of the first; of the slots in between, slot 1 of max_logits then tells the reduce
  * kernel how many partitions a partial covers (a NaN with that number in its low byte), the
- * others stay untouched.  Only `out` is a result. */
+ * others stay untouched; and a row whose whole context lies in one partial gets that partial
+ * straight into `out`, as its result -- its scalars are in exp_sums and max_logits, its tmp_out
+ * row stays untouched.  Only `out` is a result. */
 int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
                                   const void *value_cache, const int32_t *block_tables,
                                   const int32_t *context_lens, float scale,

@@ -59,6 +59,8 @@ def test_kernels_match_fixtures(golden, name):
                                        rtol=1e-5, atol=1e-4)
             np.testing.assert_allclose(bufs.exp_sums.cpu().numpy()[live], golden[f"{name}/exp_sums"][live],
                                        rtol=1e-4, atol=1e-4)
-            np.testing.assert_allclose(bufs.tmp_out.cpu().numpy()[live], golden[f"{name}/tmp_out"][live],
+            # a row of a single partial has it in `out` (as the row's result), not in tmp_out
+            several = live & (live.sum(axis=2, keepdims=True) >= 2)
+            np.testing.assert_allclose(bufs.tmp_out.cpu().numpy()[several], golden[f"{name}/tmp_out"][several],
                                        rtol=1e-2, atol=1e-2)
             assert np.isnan(bufs.exp_sums.cpu().numpy()[~live]).all()
