@@ -167,8 +167,11 @@ def _time_config(built, steps, warmup, torch, W, runner, dev, schedule=0, traffi
         longest = int(torch.argmax(w.context_lens))
         slots = torch.nonzero(written[longest, 0]).flatten().tolist()
         res["scratch_bytes_allocated"] = w.scratch_bytes()
-        res["scratch_bytes_written"] = int(written.sum()) * (D + 2) * 4
+        # a row's only partial goes into `out` as its result: two scalars in the scratch arrays, no row
+        rows = ~torch.isnan(probe.tmp_out[..., 0])
+        res["scratch_bytes_written"] = int(written.sum()) * 2 * 4 + int(rows.sum()) * D * 4
         res["partials"] = int(written.sum()) // H * w.num_kv_heads
+        res["partials_stored_into_out"] = (int(written.sum()) - int(rows.sum())) // H * w.num_kv_heads
         res["partitions_per_segment"] = (slots[1] - slots[0]) if len(slots) > 1 else None
         res["partition_size"] = w.partition_size
     return w, res
