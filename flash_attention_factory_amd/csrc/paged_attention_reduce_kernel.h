@@ -82,9 +82,6 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
     // one partial: the segment kernel has stored it into `out` as the row's result
     // (PagedAttnParams::final_out), and its tmp_out row holds nothing
     if (np == 1) return;
-#ifdef FA_X_DIRECT
-    if (np == 1) return;
-#endif
   }
   const float *ml = p.max_logits + base;
   const float *es = p.exp_sums + base;

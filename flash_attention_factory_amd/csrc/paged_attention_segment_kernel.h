@@ -159,11 +159,6 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       }
       const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
       const int d0 = wa.out_elem(4 * r * NDT + tw * SL);
-#ifdef FA_X_DIRECT
-      if (it.part0 == 0 && it.tok_end >= it.ctx)  // timing only: the row's only partial, as 16-bit values
-        W::template store_q<SL>(reinterpret_cast<char *>(p.out) + (slot * wa.out_row_elems()) * 4 + d0 * 2, o, inv);
-      else
-#endif
       // the row's only partial is its result (PagedAttnParams::final_out); it.ctx is the length as
       // far as the scratch arrays hold it
       if (p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx)
