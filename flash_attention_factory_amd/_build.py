@@ -16,40 +16,6 @@ HIPCC_FLAGS = [
 ]
 
 
-COPY_PROBE_SOURCE = os.path.join(_PKG, "csrc", "hbm_copy_probe.hip")
-COPY_PROBE = os.path.join(_PKG, "hbm_copy_probe")
-
-
-def build_copy_probe(verbose: bool = False) -> str:
-    """The plain-copy program that calibrates rocprofv3's HBM traffic counters."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", COPY_PROBE_SOURCE, "-o", COPY_PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
-    return COPY_PROBE
-
-
-STREAM_PROBE_SOURCE = os.path.join(_PKG, "csrc", "hbm_stream_probe.hip")
-STREAM_PROBE = os.path.join(_PKG, "hbm_stream_probe")
-
-
-def build_stream_probe(verbose: bool = False) -> str:
-    """The streaming probe behind the K load pattern and the no-LDS-staging choice."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", STREAM_PROBE_SOURCE, "-o", STREAM_PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
-    return STREAM_PROBE
-
-
 def build(verbose: bool = False, extra_flags=()) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, SOURCE, "-o", LIBRARY]

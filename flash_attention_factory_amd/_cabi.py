@@ -36,7 +36,10 @@ EXPORTS = (
     "fa_paged_attention_abi_version",
     "fa_kv_cache_write",
     "fa_paged_attention_reduce_static_scratch",
+    "fa_paged_attention_kernel_status",
 )
+
+ABI_REVISION = 8
 
 FA_KV_CACHE_16BIT = 0
 FA_KV_CACHE_E5M2 = 1
@@ -58,8 +61,19 @@ FA_MASK_SOFTCAP = 2
 FA_MASK_WINDOW = 4
 
 
-class Shape(ctypes.Structure):
+class _Versioned(ctypes.Structure):
+    """A struct that begins with `struct_size`: set on construction to the size declared here, which
+    is how the library knows which fields the caller's revision of the header has."""
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        if "struct_size" not in kw:
+            self.struct_size = ctypes.sizeof(type(self))
+
+
+class Shape(_Versioned):
     _fields_ = [
+        ("struct_size", ctypes.c_uint32),
         ("num_seqs", ctypes.c_int32),
         ("num_heads", ctypes.c_int32),
         ("num_kv_heads", ctypes.c_int32),
@@ -76,8 +90,9 @@ class Shape(ctypes.Structure):
     ]
 
 
-class Options(ctypes.Structure):
+class Options(_Versioned):
     _fields_ = [
+        ("struct_size", ctypes.c_uint32),
         ("sinks", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
         ("softcap", ctypes.c_float),
@@ -93,11 +108,13 @@ class Options(ctypes.Structure):
         ("k_scales", ctypes.c_void_p),
         ("v_scales", ctypes.c_void_p),
         ("schedule", ctypes.c_int32),
+        ("spin_limit", ctypes.c_int32),
     ]
 
 
-class KvWriteShape(ctypes.Structure):
+class KvWriteShape(_Versioned):
     _fields_ = [
+        ("struct_size", ctypes.c_uint32),
         ("num_tokens", ctypes.c_int32),
         ("num_kv_heads", ctypes.c_int32),
         ("head_size", ctypes.c_int32),
@@ -180,8 +197,20 @@ def load() -> ctypes.CDLL:
     L.fa_kv_cache_write.restype = ctypes.c_int32
     L.fa_last_error.restype = ctypes.c_char_p
     L.fa_paged_attention_abi_version.restype = ctypes.c_int32
+    L.fa_paged_attention_kernel_status.argtypes = [P, ctypes.c_int32]
+    L.fa_paged_attention_kernel_status.restype = ctypes.c_int32
+    if L.fa_paged_attention_abi_version() != ABI_REVISION:
+        raise RuntimeError(f"{LIBRARY} has ABI revision {L.fa_paged_attention_abi_version()}, this binding is "
+                           f"written for {ABI_REVISION}: rebuild the library")
     _lib = L
     return L
+
+
+def kernel_status(stream: int = 0, clear: bool = True) -> None:
+    """Raise PagedAttentionError if a persistent kernel of the current GPU gave up a wait since the
+    status word was last cleared (waits for `stream`, a raw hipStream_t, first).  For callers of the
+    asynchronous paths, at a synchronisation point of their own; timed calls look by themselves."""
+    check(load().fa_paged_attention_kernel_status(stream or None, 1 if clear else 0))
 
 
 def check(code: int) -> None:

@@ -20,8 +20,11 @@ FA_EXPORT int32_t fa_paged_attention_loop(void *out, const void *query, const vo
                                           int32_t max_context_len,
                                           const fa_paged_attention_shape *shape,
                                           const fa_paged_attention_options *options) {
+  fa::CallStructs c;
+  const fa_status st = fa::read_call_structs(shape, options, &c);
+  if (st != FA_OK) return st;
   return fa::dispatch_paged_attention_loop(out, query, key_cache, value_cache, block_tables,
-                                           context_lens, scale, max_context_len, shape, options);
+                                           context_lens, scale, max_context_len, &c.shape, c.options());
 }
 
 FA_EXPORT int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
@@ -31,9 +34,12 @@ FA_EXPORT int32_t fa_paged_attention_reduce(void *out, const void *query, const 
                                             float *max_logits, float *tmp_out,
                                             const fa_paged_attention_shape *shape,
                                             const fa_paged_attention_options *options) {
+  fa::CallStructs c;
+  const fa_status st = fa::read_call_structs(shape, options, &c);
+  if (st != FA_OK) return st;
   return fa::dispatch_paged_attention(out, query, key_cache, value_cache, block_tables,
                                       context_lens, scale, max_context_len, exp_sums, max_logits,
-                                      tmp_out, shape, options);
+                                      tmp_out, &c.shape, c.options());
 }
 
 // ---- the entry point that allocates nothing ---------------------------------------------
@@ -74,8 +80,11 @@ FA_EXPORT int32_t fa_paged_attention_reduce_static_scratch(void *out, const void
                                                            int32_t max_context_len,
                                                            const fa_paged_attention_shape *shape,
                                                            const fa_paged_attention_options *options) {
-  fa::error_buffer()[0] = 0;
-  if (!shape) return fa::fail(FA_ERR_NULL_POINTER, "shape is NULL");
+  fa::CallStructs c;
+  const fa_status read = fa::read_call_structs(shape, options, &c);
+  if (read != FA_OK) return read;
+  shape = &c.shape;
+  options = c.options();
   if (options && options->elapsed_us)
     return fa::fail(FA_ERR_BAD_SHAPE, "fa_paged_attention_reduce_static_scratch allocates nothing, events included: "
                                       "elapsed_us must be NULL (time the call with fa_paged_attention_reduce)");
@@ -113,9 +122,12 @@ FA_EXPORT int32_t fa_paged_attention_fp8_loop(void *out, const void *query, cons
                                               int32_t max_context_len,
                                               const fa_paged_attention_shape *shape,
                                               const fa_paged_attention_options *options) {
+  fa::CallStructs c;
+  const fa_status st = fa::read_call_structs(shape, options, &c);
+  if (st != FA_OK) return st;
   return fa::dispatch_paged_attention_fp8_loop(out, query, key_cache, value_cache, block_tables,
-                                               context_lens, scale, max_context_len, shape,
-                                               options);
+                                               context_lens, scale, max_context_len, &c.shape,
+                                               c.options());
 }
 
 FA_EXPORT int32_t fa_paged_attention_fp8_reduce(void *out, const void *query,
@@ -126,18 +138,34 @@ FA_EXPORT int32_t fa_paged_attention_fp8_reduce(void *out, const void *query,
                                                 float *max_logits, float *tmp_out,
                                                 const fa_paged_attention_shape *shape,
                                                 const fa_paged_attention_options *options) {
+  fa::CallStructs c;
+  const fa_status st = fa::read_call_structs(shape, options, &c);
+  if (st != FA_OK) return st;
   return fa::dispatch_paged_attention_fp8(out, query, key_cache, value_cache, block_tables,
                                           context_lens, scale, max_context_len, exp_sums,
-                                          max_logits, tmp_out, shape, options);
+                                          max_logits, tmp_out, &c.shape, c.options());
 }
 
 FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *key_cache,
                                     void *value_cache, const int64_t *slot_mapping,
                                     const fa_kv_cache_write_shape *shape,
                                     const fa_paged_attention_options *options) {
-  return fa::launch_kv_cache_write(key, value, key_cache, value_cache, slot_mapping, shape, options);
+  fa::error_buffer()[0] = 0;
+  if (!shape) return fa::fail(FA_ERR_NULL_POINTER, "shape is NULL");
+  fa_kv_cache_write_shape sh;
+  fa::CallStructs c;
+  constexpr size_t kLeast = offsetof(fa_kv_cache_write_shape, num_pool_blocks) + sizeof(int64_t);
+  fa_status st = fa::read_versioned(shape, &sh, kLeast, "shape");
+  if (st == FA_OK) st = fa::read_options(options, &c);
+  if (st != FA_OK) return st;
+  return fa::launch_kv_cache_write(key, value, key_cache, value_cache, slot_mapping, &sh, c.options());
+}
+
+FA_EXPORT int32_t fa_paged_attention_kernel_status(void *stream, int32_t clear) {
+  fa::error_buffer()[0] = 0;
+  return fa::read_kernel_status(reinterpret_cast<hipStream_t>(stream), clear != 0, 0);
 }
 
 FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
 
-FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return 7; }
+FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return fa::kAbiRevision; }

@@ -12,7 +12,9 @@
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stddef.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include <algorithm>
 #include <mutex>
@@ -27,6 +29,8 @@
 #include "paged_attention_segment_kernel.h"
 
 namespace fa {
+
+constexpr int kAbiRevision = 8;  // fa_paged_attention_abi_version()
 
 inline char *error_buffer() {
   static thread_local char buf[512] = {0};
@@ -73,12 +77,53 @@ inline fa_status kernel_status_of_current_device(int32_t **word) {
   return FA_OK;
 }
 
-// FA_DEBUG_SPIN_LIMIT in the environment replaces the spin limit of the persistent kernels: the way
-// to see the give-up path run (a limit of 0 makes every merge go ahead without waiting) while every
-// kernel still ends normally.
-inline int32_t spin_limit_of_this_call() {
-  const char *text = getenv("FA_DEBUG_SPIN_LIMIT");
-  return text ? (int32_t)atoi(text) : kLoopPersistentSpinLimit;
+// The spin limit of a call's persistent kernels (fa_paged_attention_options::spin_limit): 0 = the
+// library's bound, negative = no polls at all, so that every wait gives up at once -- the way to see
+// the give-up path run while every kernel still ends normally.
+inline int32_t spin_limit_of(const fa_paged_attention_options *o) {
+  if (!o || o->spin_limit == 0) return kLoopPersistentSpinLimit;
+  return o->spin_limit < 0 ? 0 : o->spin_limit;
+}
+
+// A versioned struct as the library works with it: the `struct_size` bytes the caller's header
+// knows, every later field zero.  `least`: bytes of the fields the struct cannot do without.
+template <typename T>
+inline fa_status read_versioned(const T *in, T *out, size_t least, const char *name) {
+  const size_t size = in->struct_size;
+  if (size < least || size > sizeof(T) || size % 4)
+    return fail(FA_ERR_BAD_SHAPE, "%s.struct_size is %zu: it must be sizeof of the struct in the caller's header, "
+                                  "%zu to %zu bytes for this library (ABI revision %d)",
+                name, size, least, sizeof(T), kAbiRevision);
+  memset(reinterpret_cast<char *>(out), 0, sizeof(T));
+  memcpy(reinterpret_cast<char *>(out), reinterpret_cast<const char *>(in), size);
+  out->struct_size = (uint32_t)sizeof(T);
+  return FA_OK;
+}
+
+// Shape and options of a decode entry point, copied out of the caller's structs.  options() is
+// NULL when the caller passed none.
+struct CallStructs {
+  fa_paged_attention_shape shape;
+  fa_paged_attention_options options_storage;
+  bool has_options = false;
+  const fa_paged_attention_options *options() const { return has_options ? &options_storage : nullptr; }
+};
+
+inline fa_status read_options(const fa_paged_attention_options *options, CallStructs *c) {
+  c->has_options = options != nullptr;
+  if (!options) return FA_OK;
+  return read_versioned(options, &c->options_storage, sizeof(uint32_t), "options");
+}
+
+inline fa_status read_call_structs(const fa_paged_attention_shape *shape, const fa_paged_attention_options *options,
+                                   CallStructs *c) {
+  error_buffer()[0] = 0;
+  if (!shape) return fail(FA_ERR_NULL_POINTER, "shape is NULL");
+  // every field of revision 8 is needed: the struct ends with num_pool_blocks
+  constexpr size_t kShapeLeast = offsetof(fa_paged_attention_shape, num_pool_blocks) + sizeof(int32_t);
+  const fa_status st = read_versioned(shape, &c->shape, kShapeLeast, "shape");
+  if (st != FA_OK) return st;
+  return read_options(options, c);
 }
 
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
@@ -225,30 +270,44 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->validate_only = o && o->validate_only != 0;
   r->sinks = o ? o->sinks : nullptr;
   r->status = nullptr;
-  r->spin_limit = spin_limit_of_this_call();
+  r->spin_limit = spin_limit_of(o);
   if (!r->validate_only) return kernel_status_of_current_device(&r->status);
   return FA_OK;
 }
 
-// After a timed call (which has synchronised anyway): did a kernel of this GPU give up a wait?
-// Reads the status word, clears it, and turns a set word into FA_ERR_RUNTIME.  Asynchronous calls
-// do not look: the word stays set until the next timed call on the device reports it.
-inline fa_status report_kernel_status(const Resolved &r) {
-  if (!r.elapsed_us || !r.status) return FA_OK;
+// Did a kernel of the current GPU give up a wait since the status word was last cleared?  Waits for
+// `stream`, reads the word, clears it on request, and turns a set word into FA_ERR_RUNTIME.
+inline fa_status read_kernel_status(hipStream_t stream, bool clear, int32_t spin_limit) {
+  int32_t *word = nullptr;
+  const fa_status st = kernel_status_of_current_device(&word);
+  if (st != FA_OK) return st;
   // read through one pinned word per thread (a copy into pageable memory costs ten times as much);
-  // allocated on the first timed call, like the timing events
+  // allocated on the first look, like the timing events
   static thread_local int32_t *pinned = nullptr;
   if (pinned == nullptr) FA_HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&pinned), sizeof(int32_t), hipHostMallocDefault));
-  FA_HIP_CHECK(hipMemcpyAsync(pinned, r.status, sizeof(int32_t), hipMemcpyDeviceToHost, r.stream));
-  FA_HIP_CHECK(hipStreamSynchronize(r.stream));
+  FA_HIP_CHECK(hipMemcpyAsync(pinned, word, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  FA_HIP_CHECK(hipStreamSynchronize(stream));
   const int32_t seen = *pinned;
   if (seen == 0) return FA_OK;
-  const int32_t zero = 0;
-  FA_HIP_CHECK(hipMemcpyAsync(r.status, &zero, sizeof(zero), hipMemcpyHostToDevice, r.stream));
-  FA_HIP_CHECK(hipStreamSynchronize(r.stream));
-  return fail(FA_ERR_RUNTIME, "a wavefront gave up waiting for the other wavefronts of its work-group (spin limit %d, "
-                              "status %d): the output of this or an earlier call on this GPU is not valid",
-              r.spin_limit, seen);
+  if (clear) {
+    const int32_t zero = 0;
+    FA_HIP_CHECK(hipMemcpyAsync(word, &zero, sizeof(zero), hipMemcpyHostToDevice, stream));
+    FA_HIP_CHECK(hipStreamSynchronize(stream));
+  }
+  if (spin_limit > 0)
+    return fail(FA_ERR_RUNTIME, "a wavefront gave up waiting for the other wavefronts of its work-group (spin limit %d, "
+                                "status %d): the output of this or an earlier call on this GPU is not valid",
+                spin_limit, seen);
+  return fail(FA_ERR_RUNTIME, "a wavefront gave up waiting for the other wavefronts of its work-group (status %d): the "
+                              "output of this or an earlier call on this GPU is not valid", seen);
+}
+
+// After a timed call (which has synchronised anyway): report and clear the status word.
+// Asynchronous calls do not look: the word stays set until the next timed call on the device, or
+// fa_paged_attention_kernel_status, reports it.
+inline fa_status report_kernel_status(const Resolved &r) {
+  if (!r.elapsed_us || !r.status) return FA_OK;
+  return read_kernel_status(r.stream, true, r.spin_limit);
 }
 
 inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits, const void *query,

@@ -17,9 +17,9 @@ from ._run import run_impl
 def run(max_logits, exp_sums, tem_output, output, debug_output, query, key_cache, value_cache,
         block_tables, context_lens, num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
         alibi_slopes, sinks, softcap, *, timed=True, partition_size=0, apply_alibi=False, apply_softcap=False, window_left=None, schedule=0,
-        k_scales=None, v_scales=None):
+        k_scales=None, v_scales=None, spin_limit=0):
     return run_impl("fa_paged_attention_fp8_reduce", True, True, max_logits, exp_sums, tem_output, output,
                     debug_output, query, key_cache, value_cache, block_tables, context_lens,
                     num_queries_per_tokens, sm_scale, fp8_scale, block_size, max_context_len,
                     alibi_slopes, sinks, softcap, timed=timed, partition_size=partition_size, apply_alibi=apply_alibi,
-                    apply_softcap=apply_softcap, window_left=window_left, schedule=schedule, k_scales=k_scales, v_scales=v_scales)
+                    apply_softcap=apply_softcap, window_left=window_left, schedule=schedule, k_scales=k_scales, v_scales=v_scales, spin_limit=spin_limit)

@@ -28,8 +28,10 @@ FP8 operators and ``kv_cache_write`` take ``k_scales`` / ``v_scales`` (fp32 ``[k
 SCRATCH CAPACITY of the reduce operators: ``exp_sums.size(-1)`` partitions of ``partition_size`` tokens must
 cover the longest context of the batch.  The kernels cannot raise an error: a longer context is attended
 over its first ``partitions * partition_size`` tokens only.  Pass ``max_context_len`` (the longest
-context, known on the host) and the call fails with FA_ERR_PARTITION_OVERFLOW instead; with the default
-0 nothing is checked.
+context, known on the host) and the call fails with FA_ERR_PARTITION_OVERFLOW instead.  Without it (the
+default, -1) the only bound the host has is what the block table can hold, ``block_tables.size(1) *
+block_size``: if the scratch arrays hold fewer tokens than that, a RuntimeWarning says so, once; an
+explicit 0 checks nothing and warns of nothing.
 
 Caches are ``[blocks, block_size, kv_heads, head_size]`` views as in ``lib.*.run``; every
 output is an argument the operator mutates, nothing is allocated.  Importing this module
@@ -51,6 +53,28 @@ _NS = "fa_amd"
 
 def _group(query: Tensor, key_cache: Tensor) -> int:
     return query.size(-2) // key_cache.size(2)
+
+
+_warned_capacity = False
+
+
+def _checked_context_len(max_context_len: int, exp_sums: Tensor, partition_size: int, query: Tensor,
+                         key_cache: Tensor, block_tables: Tensor) -> int:
+    """What the launcher is told the longest context is.  -1: unknown -- warn once if the block table
+    could hold a context the scratch arrays cannot (nothing is read from the device for this)."""
+    if max_context_len >= 0:
+        return max_context_len
+    global _warned_capacity
+    if not _warned_capacity:
+        size = partition_size if partition_size > 0 else (256 if query.size(-1) == 64 else 512)
+        if exp_sums.size(-1) * size < block_tables.size(1) * key_cache.size(1):
+            _warned_capacity = True
+            import warnings
+            warnings.warn(f"the scratch arrays hold {exp_sums.size(-1)} partitions of {size} tokens, the block table "
+                          f"{block_tables.size(1)} blocks of {key_cache.size(1)}: a context beyond "
+                          f"{exp_sums.size(-1) * size} tokens would be attended over its first tokens only -- pass "
+                          "max_context_len to have that checked (0 to silence this warning)", RuntimeWarning, stacklevel=3)
+    return 0
 
 
 def _modifiers(alibi_slopes: Optional[Tensor], softcap: float, window_left: int) -> dict:
@@ -85,9 +109,10 @@ def paged_attention_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor, tm
                            key_cache: Tensor, value_cache: Tensor, block_tables: Tensor, context_lens: Tensor,
                            scale: float, partition_size: int = 0, sinks: Optional[Tensor] = None,
                            alibi_slopes: Optional[Tensor] = None, softcap: float = 0.0,
-                           window_left: int = -1, max_context_len: int = 0) -> None:
+                           window_left: int = -1, max_context_len: int = -1) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
+    max_context_len = _checked_context_len(max_context_len, exp_sums, partition_size, query, key_cache, block_tables)
     _reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
                 context_lens, _group(query, key_cache), scale, key_cache.size(1), max_context_len, alibi_slopes, sinks,
                 softcap, partition_size=partition_size, timed=False, **_modifiers(alibi_slopes, softcap, window_left))
@@ -100,9 +125,10 @@ def paged_attention_fp8_reduce(out: Tensor, exp_sums: Tensor, max_logits: Tensor
                                context_lens: Tensor, scale: float, fp8_scale: float, partition_size: int = 0,
                                sinks: Optional[Tensor] = None, alibi_slopes: Optional[Tensor] = None,
                                softcap: float = 0.0, window_left: int = -1, k_scales: Optional[Tensor] = None,
-                               v_scales: Optional[Tensor] = None, max_context_len: int = 0) -> None:
+                               v_scales: Optional[Tensor] = None, max_context_len: int = -1) -> None:
     if tmp_out.dtype != torch.float32:
         raise RuntimeError("tmp_out must be fp32: these operators allocate nothing, not even a workspace")
+    max_context_len = _checked_context_len(max_context_len, exp_sums, partition_size, query, key_cache, block_tables)
     _fp8_reduce.run(max_logits, exp_sums, tmp_out, out, None, query, key_cache, value_cache, block_tables,
                     context_lens, _group(query, key_cache), scale, fp8_scale, key_cache.size(1), max_context_len,
                     alibi_slopes, sinks, softcap, partition_size=partition_size, timed=False, k_scales=k_scales,

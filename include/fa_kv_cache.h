@@ -48,6 +48,7 @@ typedef enum fa_kv_cache_dtype {
 } fa_kv_cache_dtype;
 
 typedef struct fa_kv_cache_write_shape {
+  uint32_t struct_size;     /* sizeof(fa_kv_cache_write_shape) in the caller's header */
   int32_t num_tokens;
   int32_t num_kv_heads;
   int32_t head_size;        /* multiple of 8 */
@@ -61,6 +62,7 @@ typedef struct fa_kv_cache_write_shape {
   int32_t cache_dtype;      /* fa_kv_cache_dtype */
   int64_t num_pool_blocks;  /* blocks in each pool, > 0: slots outside the pool are skipped */
 } fa_kv_cache_write_shape;
+#define FA_KV_CACHE_WRITE_SHAPE_INIT {(uint32_t)sizeof(fa_kv_cache_write_shape)}
 
 /* Of `options` this entry reads fp8_scale (FP8 pools only; 0 means 1.0), kv_scale_mode with
  * k_scales / v_scales (FP8 pools only: the byte stored is the rounding of x * (1 / scale), the

@@ -48,6 +48,14 @@
  * A sequence with context_lens[s] <= 0 leaves its rows of `out` untouched; a
  * context length above max_blocks_per_seq * block_size is cut to that bound, so the
  * kernels never read past a row of block_tables.
+ *
+ * Versioned structs.  fa_paged_attention_shape, fa_paged_attention_options and
+ * fa_kv_cache_write_shape begin with `struct_size`, which the caller sets to sizeof of the
+ * struct AS ITS HEADER DECLARES IT (the *_INIT macros do).  The library reads that many bytes and
+ * takes every later field as zero, its default, so a caller built against an older revision of
+ * this header keeps working when fields are appended; a size of 0, one that is not a multiple of
+ * 4, one smaller than the fields a struct cannot do without (the shapes: all fields of revision 8;
+ * the options: struct_size alone) or one larger than the library knows is FA_ERR_BAD_SHAPE.
  */
 #ifndef FA_PAGED_ATTENTION_H_
 #define FA_PAGED_ATTENTION_H_
@@ -113,6 +121,7 @@ typedef enum fa_kv_scale { FA_KV_SCALE_TENSOR = 0, FA_KV_SCALE_HEAD = 1, FA_KV_S
 /* Shapes and strides that upstream reads off the torch tensors
  * (paged_attention_loop.cpp:60-65) or fixes at compile time. */
 typedef struct fa_paged_attention_shape {
+  uint32_t struct_size;       /* sizeof(fa_paged_attention_shape) in the caller's header */
   int32_t num_seqs;
   int32_t num_heads;
   int32_t num_kv_heads;
@@ -131,10 +140,12 @@ typedef struct fa_paged_attention_shape {
                                  corrupt table cannot make the kernel touch memory outside the pool
                                  (upstream has no such guard) */
 } fa_paged_attention_shape;
+#define FA_PAGED_ATTENTION_SHAPE_INIT {(uint32_t)sizeof(fa_paged_attention_shape)}
 
 /* Everything upstream's `run` takes beyond the result-affecting list, plus stream
  * and timing control.  A NULL options pointer means all defaults. */
 typedef struct fa_paged_attention_options {
+  uint32_t struct_size;       /* sizeof(fa_paged_attention_options) in the caller's header */
   const void *sinks;          /* device, [num_heads] in q_dtype, or NULL */
   const float *alibi_slopes;  /* device, [num_heads] fp32; ignored unless FA_MASK_ALIBI */
   float softcap;              /* ignored unless FA_MASK_SOFTCAP (then > 0) */
@@ -167,7 +178,13 @@ typedef struct fa_paged_attention_options {
   const float *k_scales;      /* device, fp32, shaped as kv_scale_mode says; NULL with mode 0 */
   const float *v_scales;
   int32_t schedule;           /* fa_schedule; 0 = the library chooses */
+  int32_t spin_limit;         /* persistent kernels: polls a wavefront spends on one wait for the other
+                                 wavefronts of its work-group before it gives up (and the call's result is
+                                 void, see fa_paged_attention_kernel_status).  0 = the library's bound,
+                                 which no correct run reaches; negative = do not wait at all, which makes
+                                 the give-up path run for a test while every kernel still ends normally */
 } fa_paged_attention_options;
+#define FA_PAGED_ATTENTION_OPTIONS_INIT {(uint32_t)sizeof(fa_paged_attention_options)}
 
 /* Single-pass kernel: no scratch.  One launch for a decode batch of up to 128 sequences; larger
  * batches and query blocks of more than 32 (token, head) columns per kv head take several. */
@@ -235,7 +252,17 @@ int32_t fa_paged_attention_fp8_reduce(void *out, const void *query, const void *
 /* Text of the last failure on the calling thread ("" if none). */
 const char *fa_last_error(void);
 
-/* ABI revision of this header. */
+/* Did a persistent kernel of the current GPU give up a wait for the wavefronts of its work-group
+ * (options->spin_limit) since the word was last cleared?  Then the output of that call is not
+ * valid.  Timed calls (elapsed_us) look by themselves and return FA_ERR_RUNTIME; asynchronous
+ * calls cannot, so their caller asks here at a synchronisation point of its own: the function
+ * waits for `stream` (a hipStream_t; NULL = the null stream), reads the word and, with `clear`
+ * non-zero, resets it.  Returns FA_OK (nothing happened) or FA_ERR_RUNTIME with the reason in
+ * fa_last_error().  One word per GPU: it does not say which call it was.  No counterpart upstream
+ * (whose work-groups meet at barriers, paged_attention_kernel_loop.hpp:345-347). */
+int32_t fa_paged_attention_kernel_status(void *stream, int32_t clear);
+
+/* ABI revision of this header: 8 (structs begin with struct_size). */
 int32_t fa_paged_attention_abi_version(void);
 
 #ifdef __cplusplus

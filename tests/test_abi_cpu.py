@@ -29,22 +29,95 @@ def test_header_symbols_are_exported(L):
     assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
-    assert L.fa_paged_attention_abi_version() == 7
+    assert L.fa_paged_attention_abi_version() == 8 == _cabi.ABI_REVISION
 
 
 def test_struct_layouts_match_header():
-    # field order and sizes of the two structs as the header lays them out
-    assert ctypes.sizeof(_cabi.Shape) == 8 * 4 + 3 * 8 + 2 * 4
-    assert _cabi.Shape.kv_block_stride.offset == 32
-    assert ctypes.sizeof(_cabi.Options) == 8 + 8 + 4 + 4 + 8 + 8 + 4 + 4 + 4 + 4 + 4 + 4 + 8 + 8 + 8
-    assert _cabi.Options.schedule.offset == 80
-    assert _cabi.Options.kv_scale_mode.offset == 60
-    assert _cabi.Options.k_scales.offset == 64 and _cabi.Options.v_scales.offset == 72
-    assert _cabi.Options.query_len.offset == 56
-    assert _cabi.Options.mask_flags.offset == 48 and _cabi.Options.window_left.offset == 52
-    assert _cabi.Options.elapsed_us.offset == 32
-    assert ctypes.sizeof(_cabi.KvWriteShape) == 4 * 4 + 5 * 8 + 2 * 4 + 8
-    assert _cabi.KvWriteShape.src_dtype.offset == 56 and _cabi.KvWriteShape.num_pool_blocks.offset == 64
+    # field order and sizes of the three structs as the headers lay them out (revision 8: every
+    # struct begins with struct_size)
+    assert _cabi.Shape.struct_size.offset == 0 and _cabi.Shape.num_seqs.offset == 4
+    assert ctypes.sizeof(_cabi.Shape) == 4 + 8 * 4 + 4 + 3 * 8 + 2 * 4 == 72
+    assert _cabi.Shape.kv_block_stride.offset == 40
+    assert _cabi.Shape.num_pool_blocks.offset == 68
+    assert _cabi.Options.struct_size.offset == 0 and _cabi.Options.sinks.offset == 8
+    assert ctypes.sizeof(_cabi.Options) == 96
+    assert _cabi.Options.schedule.offset == 88 and _cabi.Options.spin_limit.offset == 92
+    assert _cabi.Options.kv_scale_mode.offset == 68
+    assert _cabi.Options.k_scales.offset == 72 and _cabi.Options.v_scales.offset == 80
+    assert _cabi.Options.query_len.offset == 64
+    assert _cabi.Options.mask_flags.offset == 56 and _cabi.Options.window_left.offset == 60
+    assert _cabi.Options.elapsed_us.offset == 40
+    assert ctypes.sizeof(_cabi.KvWriteShape) == 4 + 4 * 4 + 4 + 5 * 8 + 2 * 4 + 8 == 80
+    assert _cabi.KvWriteShape.src_dtype.offset == 64 and _cabi.KvWriteShape.num_pool_blocks.offset == 72
+    # a new struct says how large it is
+    assert _cabi.Shape().struct_size == 72 and _cabi.Options().struct_size == 96 and _cabi.KvWriteShape().struct_size == 80
+
+
+def test_header_struct_sizes_agree_with_the_compiler(tmp_path):
+    """The headers as a C compiler lays them out: sizes and the offsets the binding relies on."""
+    import subprocess
+    src = tmp_path / "sizes.c"
+    src.write_text(
+        '#include <stddef.h>\n#include <stdio.h>\n#include "fa_kv_cache.h"\n'
+        'int main(void) {\n'
+        '  fa_paged_attention_shape s = FA_PAGED_ATTENTION_SHAPE_INIT;\n'
+        '  fa_paged_attention_options o = FA_PAGED_ATTENTION_OPTIONS_INIT;\n'
+        '  fa_kv_cache_write_shape k = FA_KV_CACHE_WRITE_SHAPE_INIT;\n'
+        '  printf("%u %u %u %zu %zu %zu %zu %d\\n", s.struct_size, o.struct_size, k.struct_size,\n'
+        '         offsetof(fa_paged_attention_shape, num_pool_blocks), offsetof(fa_paged_attention_options, schedule),\n'
+        '         offsetof(fa_paged_attention_options, spin_limit), offsetof(fa_kv_cache_write_shape, num_pool_blocks),\n'
+        '         s.num_seqs + o.schedule + k.num_tokens);\n'
+        '  return 0;\n}\n')
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert [int(x) for x in out] == [72, 96, 80, 68, 88, 92, 72, 0]
+
+
+def test_shorter_and_longer_structs(L):
+    """struct_size tells the library which fields the caller's header has: an options struct cut
+    before `schedule` (a caller built before the field was appended) validates with the field at its
+    default; sizes the library cannot make sense of are refused."""
+    def call(shape_size=None, options_size=None, schedule=0, kv=False):
+        op = _cabi.Options()
+        op.validate_only = 1
+        op.schedule = schedule
+        if options_size is not None:
+            op.struct_size = options_size
+        p = 0x1000
+        if kv:
+            sh = _cabi.KvWriteShape()
+            for k, v in dict(num_tokens=4, num_kv_heads=2, head_size=128, block_size=16, kv_block_stride=2 * 16 * 128,
+                             kv_token_stride=128, kv_head_stride=16 * 128, src_dtype=0, cache_dtype=1, num_pool_blocks=8).items():
+                setattr(sh, k, v)
+            if shape_size is not None:
+                sh.struct_size = shape_size
+            return L.fa_kv_cache_write(p, p, p, p, p, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
+        sh = _shape()
+        if shape_size is not None:
+            sh.struct_size = shape_size
+        return L.fa_paged_attention_loop(p, p, p, p, p, p, 0.1, 0, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
+
+    assert call() == (_cabi.FA_OK, "")
+    assert call(schedule=3)[0] == _cabi.FA_ERR_BAD_SHAPE                      # the field is read ...
+    before_schedule = _cabi.Options.schedule.offset
+    assert call(options_size=before_schedule, schedule=3) == (_cabi.FA_OK, "")  # ... unless the caller's struct ends before it
+    assert call(options_size=_cabi.Options.spin_limit.offset, schedule=3)[0] == _cabi.FA_ERR_BAD_SHAPE
+    # the shortest struct this test may pass ends with validate_only (without it the call would launch)
+    assert call(options_size=_cabi.Options.validate_only.offset + 4, schedule=3) == (_cabi.FA_OK, "")
+    for bad in (0, 2, 97, 100, 1 << 20):
+        rc, msg = call(options_size=bad)
+        assert rc == _cabi.FA_ERR_BAD_SHAPE and "options.struct_size" in msg, (bad, msg)
+    for bad in (0, 36, 68, 70, 76, 4096):  # every field of the shape is needed
+        rc, msg = call(shape_size=bad)
+        assert rc == _cabi.FA_ERR_BAD_SHAPE and "shape.struct_size" in msg, (bad, msg)
+    assert call(kv=True) == (_cabi.FA_OK, "")
+    for bad in (0, 72, 84):
+        rc, msg = call(kv=True, shape_size=bad)
+        assert rc == _cabi.FA_ERR_BAD_SHAPE and "shape.struct_size" in msg, (bad, msg)
+    rc, msg = call(kv=True, options_size=0)
+    assert rc == _cabi.FA_ERR_BAD_SHAPE and "options.struct_size" in msg
 
 
 def _shape(**kw):

@@ -23,11 +23,12 @@ def _dev():
     return torch.device("cuda:0")
 
 
-def _run(w_cpu, kernel, max_context_len=None, schedule=0, **kw):
+def _run(w_cpu, kernel, max_context_len=None, schedule=0, spin_limit=0, timed=True, **kw):
     from flash_attention_factory_amd import runner
     w = w_cpu.to(_dev())
     bufs = runner.alloc_buffers(w, **kw)
-    times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len, schedule=schedule)
+    times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len, schedule=schedule,
+                                spin_limit=spin_limit, timed=timed)
     torch.cuda.synchronize()
     return bufs, times
 
@@ -750,20 +751,24 @@ def test_seventy_thousand_sequences(oracle):
 
 def test_exhausted_spin_limit_is_reported(oracle):
     """A wavefront of a persistent kernel that gives up waiting for its work-group sets a status word
-    and lets the grid drain; the timed call returns FA_ERR_RUNTIME.  FA_DEBUG_SPIN_LIMIT = 0 makes
-    every merge go ahead without waiting, so every kernel still ends normally."""
+    and lets the grid drain; the timed call returns FA_ERR_RUNTIME.  A negative options->spin_limit
+    makes every wait give up at once (the merges go ahead without waiting, so every kernel still ends
+    normally): the very first call reports.  An asynchronous call cannot look; its caller asks
+    fa_paged_attention_kernel_status at a synchronisation point of its own."""
     from flash_attention_factory_amd import _cabi
     w = W.make_config(1, num_seqs=4, pool_blocks=512)
-    try:
-        os.environ["FA_DEBUG_SPIN_LIMIT"] = "0"
-        for kernel in ("loop", "reduce"):
-            with pytest.raises(_cabi.PagedAttentionError, match="gave up waiting") as e:
-                for _ in range(20):  # whether a wavefront finds the others' states missing is a matter of timing
-                    _run(w, kernel)
-            assert e.value.code == _cabi.FA_ERR_RUNTIME
-    finally:
-        del os.environ["FA_DEBUG_SPIN_LIMIT"]
-    for kernel in ("loop", "reduce"):  # the word was cleared with the report
+    for kernel in ("loop", "reduce"):
+        with pytest.raises(_cabi.PagedAttentionError, match="gave up waiting") as e:
+            _run(w, kernel, spin_limit=-1)
+        assert e.value.code == _cabi.FA_ERR_RUNTIME
+        _cabi.kernel_status()  # the word was cleared with the report
+        _run(w, kernel, spin_limit=-1, timed=False)  # asynchronous: nothing is raised here ...
+        with pytest.raises(_cabi.PagedAttentionError, match="gave up waiting"):
+            _cabi.kernel_status(clear=False)  # ... the caller finds out when it asks
+        with pytest.raises(_cabi.PagedAttentionError, match="gave up waiting"):
+            _cabi.kernel_status(clear=True)
+        _cabi.kernel_status()
+    for kernel in ("loop", "reduce"):
         bufs, _ = _run(w, kernel)
         _check(bufs.out, w, oracle, f"{w.name}/{kernel} after the report")
 
