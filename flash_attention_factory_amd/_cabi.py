@@ -37,6 +37,7 @@ EXPORTS = (
     "fa_kv_cache_write",
     "fa_paged_attention_reduce_static_scratch",
     "fa_paged_attention_kernel_status",
+    "fa_paged_attention_reduce_plan",
 )
 
 ABI_REVISION = 8
@@ -55,6 +56,10 @@ FA_KV_SCALE_BLOCK = 2
 FA_SCHEDULE_AUTO = 0
 FA_SCHEDULE_GRID = 1
 FA_SCHEDULE_GRID_LDS = 2
+
+FA_SPLIT_FORM_GRID = 0
+FA_SPLIT_FORM_SEGMENT = 1
+FA_SPLIT_FORM_LOOP = 2
 
 FA_MASK_ALIBI = 1
 FA_MASK_SOFTCAP = 2
@@ -109,6 +114,7 @@ class Options(_Versioned):
         ("v_scales", ctypes.c_void_p),
         ("schedule", ctypes.c_int32),
         ("spin_limit", ctypes.c_int32),
+        ("segment_partitions", ctypes.c_int32),
     ]
 
 
@@ -127,6 +133,16 @@ class KvWriteShape(_Versioned):
         ("src_dtype", ctypes.c_int32),
         ("cache_dtype", ctypes.c_int32),
         ("num_pool_blocks", ctypes.c_int64),
+    ]
+
+
+class SplitPlan(_Versioned):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("form", ctypes.c_int32),
+        ("compute_units", ctypes.c_int32),
+        ("work_groups", ctypes.c_int32),
+        ("kv_heads_per_item", ctypes.c_int32),
     ]
 
 
@@ -197,6 +213,9 @@ def load() -> ctypes.CDLL:
     L.fa_kv_cache_write.restype = ctypes.c_int32
     L.fa_last_error.restype = ctypes.c_char_p
     L.fa_paged_attention_abi_version.restype = ctypes.c_int32
+    L.fa_paged_attention_reduce_plan.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(Options), ctypes.c_int32,
+                                                 ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(SplitPlan)]
+    L.fa_paged_attention_reduce_plan.restype = ctypes.c_int32
     L.fa_paged_attention_kernel_status.argtypes = [P, ctypes.c_int32]
     L.fa_paged_attention_kernel_status.restype = ctypes.c_int32
     if L.fa_paged_attention_abi_version() != ABI_REVISION:

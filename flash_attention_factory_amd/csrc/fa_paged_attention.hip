@@ -161,6 +161,43 @@ FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *ke
   return fa::launch_kv_cache_write(key, value, key_cache, value_cache, slot_mapping, &sh, c.options());
 }
 
+FA_EXPORT int32_t fa_paged_attention_reduce_plan(const fa_paged_attention_shape *shape,
+                                                 const fa_paged_attention_options *options, int32_t max_context_len,
+                                                 int32_t kv_fp8, int32_t compute_units, fa_split_plan *plan) {
+  fa::CallStructs c;
+  fa_status st = fa::read_call_structs(shape, options, &c);
+  if (st != FA_OK) return st;
+  if (!plan) return fa::fail(FA_ERR_NULL_POINTER, "plan is NULL");
+  if (plan->struct_size != sizeof(fa_split_plan))
+    return fa::fail(FA_ERR_BAD_SHAPE, "plan.struct_size is %u, this library's fa_split_plan has %zu bytes",
+                    plan->struct_size, sizeof(fa_split_plan));
+  // the checks of a call, made on placeholders: nothing is launched and no pointer is followed
+  static float placeholder[4] __attribute__((aligned(16)));
+  fa_paged_attention_options op = c.has_options ? c.options_storage : fa_paged_attention_options{};
+  op.struct_size = sizeof(op);
+  op.elapsed_us = nullptr;
+  void *any = placeholder;
+  const int32_t *ints = reinterpret_cast<const int32_t *>(placeholder);
+  plan->form = plan->work_groups = plan->kv_heads_per_item = 0;
+  plan->compute_units = compute_units;
+  if (compute_units > 0) {  // without a device: the form alone
+    op.validate_only = 1;
+    fa::Resolved r;
+    st = fa::validate_and_resolve(any, any, any, any, ints, ints, max_context_len, placeholder, placeholder, placeholder,
+                                  &c.shape, &op, kv_fp8 != 0, /*split=*/true, &r);
+    if (st != FA_OK) return st;
+    plan->form = fa::split_form_of(c.shape, r, kv_fp8 != 0, max_context_len, compute_units);
+    return FA_OK;
+  }
+  // with the current device: the launchers themselves, told to fill in the plan where they would launch
+  op.validate_only = 0;
+  if (kv_fp8)
+    return fa::dispatch_paged_attention_fp8(any, any, any, any, ints, ints, 1.f, max_context_len, placeholder, placeholder,
+                                            placeholder, &c.shape, &op, plan);
+  return fa::dispatch_paged_attention(any, any, any, any, ints, ints, 1.f, max_context_len, placeholder, placeholder,
+                                      placeholder, &c.shape, &op, plan);
+}
+
 FA_EXPORT int32_t fa_paged_attention_kernel_status(void *stream, int32_t clear) {
   fa::error_buffer()[0] = 0;
   return fa::read_kernel_status(reinterpret_cast<hipStream_t>(stream), clear != 0, 0);

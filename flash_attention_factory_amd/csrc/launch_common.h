@@ -153,6 +153,7 @@ struct Resolved {
   const float *k_scales;
   const float *v_scales;
   int32_t schedule;  // fa_schedule
+  int32_t segment_partitions;  // > 0: partitions per partial of the segment form, fixed by the caller
   bool pair_heads;   // two adjacent kv heads with 64-byte token rows run as one (WaveAttn::kPairable)
   int32_t *status;   // status word of the current device (nullptr with validate_only)
   int32_t spin_limit;
@@ -160,6 +161,7 @@ struct Resolved {
   float *elapsed_us;
   bool validate_only;
   const void *sinks;
+  fa_split_plan *plan;  // non-NULL: the split launcher fills this in where it would launch, and launches nothing
 };
 
 // Checks every argument the kernels rely on.  `kv8` selects byte caches, `split`
@@ -262,6 +264,8 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->schedule = o ? o->schedule : FA_SCHEDULE_AUTO;
   if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS)
     return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2)", r->schedule);
+  r->segment_partitions = o ? o->segment_partitions : 0;
+  if (r->segment_partitions < 0) return fail(FA_ERR_BAD_SHAPE, "segment_partitions must be >= 0");
   r->pair_heads = kPairHeads && kv8 && s->head_size == 64 && s->kv_head_stride == s->head_size &&
                   s->num_kv_heads % 2 == 0 && 2 * r->group <= kMaxGroup && r->mask_flags == 0 &&
                   r->query_len == 1 && r->kv_scale_mode == FA_KV_SCALE_TENSOR;
@@ -269,6 +273,7 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->elapsed_us = o ? o->elapsed_us : nullptr;
   r->validate_only = o && o->validate_only != 0;
   r->sinks = o ? o->sinks : nullptr;
+  r->plan = nullptr;
   r->status = nullptr;
   r->spin_limit = spin_limit_of(o);
   if (!r->validate_only) return kernel_status_of_current_device(&r->status);
@@ -354,6 +359,7 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
   p.compute_units = 0;  // the split path's launcher fills it in
   p.final_out = nullptr;  // (and this, in the segment form)
   p.kv_rows_apart = s.kv_token_stride != s.head_size;
+  p.segment_force = r.segment_partitions;
   p.pair_heads = 0;
   if (r.pair_heads) {  // the kernel sees pairs of kv heads: half as many, twice the group, rows of two heads
     p.pair_heads = 1;
@@ -362,6 +368,23 @@ inline PagedAttnParams make_params(void *out, float *exp_sums, float *max_logits
     p.kv_head_bytes *= 2;
   }
   return p;
+}
+
+// Compute units of the current device (asked once per thread and device).
+inline hipError_t compute_units_of_current_device(int *cus_out) {
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev != cached_dev) {
+    int cus = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    cached_dev = dev;
+    cached_cus = cus;
+  }
+  *cus_out = cached_cus;
+  return hipSuccess;
 }
 
 // How many work-groups of `threads` threads of a kernel the current device keeps resident

@@ -16,10 +16,11 @@ inline fa_status dispatch_paged_attention_fp8(void *out, const void *query, cons
                                               int32_t max_context_len, float *exp_sums,
                                               float *max_logits, float *tmp_out,
                                               const fa_paged_attention_shape *shape,
-                                              const fa_paged_attention_options *options) {
+                                              const fa_paged_attention_options *options,
+                                              fa_split_plan *plan = nullptr) {
   return dispatch_paged_attention_any<true>(out, query, key_cache, value_cache, block_tables,
                                             context_lens, scale, max_context_len, exp_sums,
-                                            max_logits, tmp_out, shape, options);
+                                            max_logits, tmp_out, shape, options, plan);
 }
 
 }  // namespace fa

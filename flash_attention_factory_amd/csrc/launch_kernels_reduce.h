@@ -12,8 +12,72 @@
 #include <algorithm>
 
 #include "launch_common.h"
+#include "launch_kernels_loop.h"
 
 namespace fa {
+
+// ---- which kernels a call of the split path runs ------------------------------------------------
+// Upstream's split path always runs its two kernels (launch_kernels_reduce.h:18-78), and its own perf
+// loop runs it on rows of 1500 keys (test_paged.py:607-631), where splitting has nothing to give: the
+// second kernel costs 4-5 us of every call whatever it finds to do, and a row of a thousand keys is
+// read by one work-group in little more than that.  What the host knows of a batch without reading
+// device memory is an upper bound on its rows: max_context_len (upstream passes seqlen_k), the block
+// table's width and the scratch arrays' capacity.  Measured over 150 batches (head sizes 64 and 128,
+// 16-bit and byte caches, 2 to 128 sequences of up to 4096 keys, equal and ragged lengths), the loop
+// kernel against the split kernels at their best segment length:
+//   rows of at most kSplitNeverBelowTokens keys        the loop kernel is as fast or faster in every
+//                                                      batch (1.0-1.9 times)
+//   rows of at most kSplitFullGpuBelowTokens keys,     faster in 26 of 30 batches (by 2-21 %; slower
+//   and a (sequence, kv head) row for every unit       by 6 and 18 % in two ragged ones)
+//   anything longer, or fewer rows                     the split kernels win, up to 2.7 times
+// In the first two cases the call IS the loop kernel: one launch, the same `out`, the scratch
+// arrays untouched, and {t, 0} as its two times.
+constexpr int kSplitNeverBelowTokens = 1024;
+constexpr int kSplitFullGpuBelowTokens = 2048;
+
+// Upper bound on the keys of a row as far as the host knows it; the scratch arrays hold
+// max_num_partitions * partition_size of them, and a call whose rows could exceed that is left to
+// the split kernels (which cut such a row to what the arrays hold).
+inline int64_t split_row_bound(const fa_paged_attention_shape &shape, int32_t partition_size, int32_t max_context_len) {
+  const int64_t table = (int64_t)shape.max_blocks_per_seq * shape.block_size;
+  const int64_t known = max_context_len > 0 ? std::min<int64_t>(max_context_len, table) : table;
+  const int64_t scratch = (int64_t)shape.max_num_partitions * partition_size;
+  return known <= scratch ? known : INT64_MAX;
+}
+
+// rows: (sequence, kv head) items as the loop kernel deals them (pairs or teams of kv heads count once)
+inline bool split_call_runs_as_loop(int64_t row_bound, int64_t rows, int compute_units) {
+  if (row_bound <= kSplitNeverBelowTokens) return true;
+  return row_bound <= kSplitFullGpuBelowTokens && rows >= compute_units;
+}
+
+// (sequence, kv head) items of a batch as the persistent loop kernel deals them.
+inline int64_t loop_rows_of(const fa_paged_attention_shape &shape, const Resolved &r, bool kv8) {
+  int64_t heads = r.pair_heads ? shape.num_kv_heads / 2 : shape.num_kv_heads;
+  // teams: two adjacent kv heads with 128-byte token rows per work-group (launch_kernels_loop.h)
+  const bool rows_128 = shape.head_size * (kv8 ? 1 : 2) == 128;
+  if (!r.pair_heads && rows_128 && shape.kv_token_stride != shape.head_size && shape.kv_head_stride == shape.head_size &&
+      shape.num_kv_heads % 2 == 0)
+    heads /= 2;
+  return (int64_t)shape.num_seqs * heads;
+}
+
+enum SplitForm { kSplitFormGrid = 0, kSplitFormSegment = 1, kSplitFormLoop = 2 };  // = fa_split_form
+
+// compute_units: of the GPU the call would run on
+inline SplitForm split_form_of(const fa_paged_attention_shape &shape, const Resolved &r, bool kv8,
+                               int32_t max_context_len, int compute_units) {
+  if (r.schedule != FA_SCHEDULE_AUTO) return kSplitFormGrid;
+  const bool loop_persistent = loop_persistent_fits(shape) && shape.num_seqs <= kLoopPersistentMaxSeqs;
+  if (loop_persistent && r.segment_partitions == 0 &&
+      split_call_runs_as_loop(split_row_bound(shape, r.partition_size, max_context_len), loop_rows_of(shape, r, kv8),
+                              compute_units))
+    return kSplitFormLoop;
+  const bool segment = (kv8 ? SegmentSplit<true>::use : SegmentSplit<false>::use) && shape.num_pool_blocks > 0 &&
+                       r.partition_size < kSegmentMaxContext &&
+                       (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
+  return segment ? kSplitFormSegment : kSplitFormGrid;
+}
 
 // Attention and reduce launches of one batch that a single attention launch can take (segment
 // form for up to kSegmentMaxSeqs sequences, else the grid form).  Kernel times are ADDED to
@@ -106,7 +170,14 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
             (int64_t)shape.num_seqs * shape.max_num_partitions * p.num_kv_heads;
         segment_groups = (int)std::min<int64_t>(resident, max_items);
       }
+      if (r.plan) {
+        r.plan->work_groups = segment_groups;
+        r.plan->kv_heads_per_item = (head_teams || r.pair_heads) ? 2 : 1;
+        return FA_OK;
+      }
       FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)segment_groups), dim3(SW * 64), 0, p));
+    } else if (r.plan) {
+      return FA_OK;
     } else if (KV8 && HEAD_SIZE == 128 && !ext && !r.pair_heads && r.schedule == FA_SCHEDULE_GRID_LDS) {
       // grid form, K and V staged through LDS: one wavefront per partition
       if constexpr (KV8 && HEAD_SIZE == 128) {
@@ -195,10 +266,25 @@ template <int HEAD_SIZE, typename QT, int KVF>
 inline fa_status launch_paged_attn_v2(void *out, const void *query, const void *key_cache,
                                       const void *value_cache, const int32_t *block_tables,
                                       const int32_t *context_lens, float scale,
-                                      int32_t /*max_context_len: validation only*/,
+                                      int32_t max_context_len,
                                       float *exp_sums, float *max_logits, float *tmp_out,
                                       const fa_paged_attention_shape &shape, const Resolved &r) {
   float us[2] = {0.f, 0.f};
+  // rows too short for splitting to pay: the call is the loop kernel (see split_call_runs_as_loop)
+  int cus = 0;
+  FA_HIP_CHECK(compute_units_of_current_device(&cus));
+  const SplitForm form = split_form_of(shape, r, KVF != kKv16, max_context_len, cus);
+  if (r.plan) {
+    r.plan->form = form;
+    r.plan->compute_units = cus;
+    if (form != kSplitFormSegment) return FA_OK;
+  }
+  if (form == kSplitFormLoop) {
+    const fa_status st = launch_paged_attn_loop<HEAD_SIZE, QT, KVF>(out, query, key_cache, value_cache, block_tables,
+                                                                    context_lens, scale, max_context_len, shape, r);
+    if (r.elapsed_us) r.elapsed_us[1] = 0.f;
+    return st;
+  }
   // most sequences one launch takes: what the segment kernel lists, or what the grid's third
   // dimension holds
   constexpr int kGridMaxSeqs = 65535;
@@ -242,12 +328,14 @@ inline fa_status dispatch_paged_attention_any(void *out, const void *query, cons
                                               int32_t max_context_len, float *exp_sums,
                                               float *max_logits, float *tmp_out,
                                               const fa_paged_attention_shape *shape,
-                                              const fa_paged_attention_options *options) {
+                                              const fa_paged_attention_options *options,
+                                              fa_split_plan *plan = nullptr) {
   Resolved r;
   fa_status st = validate_and_resolve(out, query, key_cache, value_cache, block_tables, context_lens,
                                       max_context_len, exp_sums, max_logits, tmp_out, shape, options,
                                       KV8, /*split=*/true, &r);
   if (st != FA_OK || r.validate_only) return st;
+  r.plan = plan;
   const bool bf16 = shape->q_dtype == FA_DTYPE_BF16;
 #define FA_V2_CASE(HS, QT)                                                                       \
   do {                                                                                           \
@@ -281,10 +369,11 @@ inline fa_status dispatch_paged_attention(void *out, const void *query, const vo
                                           int32_t max_context_len, float *exp_sums,
                                           float *max_logits, float *tmp_out,
                                           const fa_paged_attention_shape *shape,
-                                          const fa_paged_attention_options *options) {
+                                          const fa_paged_attention_options *options,
+                                          fa_split_plan *plan = nullptr) {
   return dispatch_paged_attention_any<false>(out, query, key_cache, value_cache, block_tables,
                                              context_lens, scale, max_context_len, exp_sums,
-                                             max_logits, tmp_out, shape, options);
+                                             max_logits, tmp_out, shape, options, plan);
 }
 
 }  // namespace fa

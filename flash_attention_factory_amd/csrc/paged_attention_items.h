@@ -114,15 +114,19 @@ struct SegmentItems {
 
   // Lane holds sequences lane, lane + 64, ...  m, the partitions per segment, follows from the
   // batch, the number of work-groups and the compute units they share (partitions_per_segment).
-  // heads_per_item: adjacent kv heads that one work-group takes together (its wavefronts in teams)
-  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane_, int groups, int heads_per_item = 1) {
+  // heads_per_item: adjacent kv heads that one work-group takes together (its wavefronts in teams);
+  // item_row_bytes: bytes of one token's K row (as of its V row) of an item
+  __device__ __forceinline__ void build(const PagedAttnParams &p, int lane_, int groups, int heads_per_item,
+                                        int item_row_bytes) {
     lane = lane_;
     S = p.num_seqs;
     Hk = p.num_kv_heads / heads_per_item;
     const int max_ctx = p.max_blocks_per_seq << p.block_shift;
     const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size, p.max_num_partitions, lane, ctxv, parts);
-    m = partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups, p.compute_units,
-                                   p.kv_rows_apart != 0);
+    m = p.segment_force > 0 ? min(p.segment_force, kSegmentMaxPartitions)
+                            : partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups,
+                                                         p.compute_units, p.kv_rows_apart != 0,
+                                                         2 * p.partition_size * item_row_bytes);
     seg_tokens = m * p.partition_size;
     int running = 0, tails = 0;
 #pragma unroll

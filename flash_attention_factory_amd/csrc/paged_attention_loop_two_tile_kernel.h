@@ -67,7 +67,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   const int r = wa.r, i = wa.i;
   using Item = WorkItem;
   std::conditional_t<PART, SegmentItems, LoopItems<TPC>> items;
-  if constexpr (PART) items.build(p, lane, G, HPW);
+  if constexpr (PART) items.build(p, lane, G, HPW, W::ROWB * HPW);
   else items.build(p, lane, tw, G, CT, HPW);
   // n-th item of this work-group, read from its first chunk that some query token of the launch
   // sees (local window; the launch's earliest query token decides: the same for both tiles)

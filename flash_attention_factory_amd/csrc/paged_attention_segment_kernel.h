@@ -68,7 +68,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   // come out even although a work-group only gets a handful of segments.
   using Item = WorkItem;  // c_lo .. c_end: the segment's chunks; ctx: the sequence's length (EXT)
   SegmentItems items;
-  items.build(p, lane, G, HPW);
+  items.build(p, lane, G, HPW, W::ROWB * HPW);
   // n-th item of this work-group; with HPW > 1 an item is HPW adjacent kv heads of one segment, of
   // which this wavefront's team takes one (kvh is then the team's own head)
   auto item_at = [&](int nth, Item &it) {

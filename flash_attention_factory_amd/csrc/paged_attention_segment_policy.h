@@ -17,6 +17,12 @@ constexpr int kSegmentMaxContext = 1 << 23;  // lengths are packed into 23 bits 
 #define FA_SEGMENT_MAX_PARTS 64
 #endif
 constexpr int kSegmentMaxPartitions = FA_SEGMENT_MAX_PARTS;
+// Where work-groups share a compute unit and each should have work throughout (see `halves` below):
+// bytes of K and V that a unit must have per segment it is given.
+#ifndef FA_SEGMENT_BYTES_WORTH_CUTTING
+#define FA_SEGMENT_BYTES_WORTH_CUTTING (768 << 10)
+#endif
+constexpr int kSegmentBytesWorthCutting = FA_SEGMENT_BYTES_WORTH_CUTTING;
 
 // a / b for 0 <= a < 2^24 and b >= 1, given inv_b close to 1 / b: both are exact in fp32, so the
 // product is off by one at most, which the remainder tells.
@@ -105,7 +111,8 @@ __device__ __forceinline__ void count_segments(const int (&ctxv)[NQ], const int 
 template <int NQ>
 __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], const int (&parts)[NQ],
                                                       int total_partitions, int S, int partition_size,
-                                                      int num_kv_heads, int groups, int cus, bool rows_apart) {
+                                                      int num_kv_heads, int groups, int cus, bool rows_apart,
+                                                      int partition_bytes) {
   const int units = max(1, min(groups, cus));  // compute units at work
   const int sharing = groups <= units ? 1 : groups <= 2 * units ? 2 : (groups + units - 1) / units;  // work-groups on each
   int live = 0;
@@ -125,8 +132,15 @@ __device__ __forceinline__ int partitions_per_segment(const int (&ctxv)[NQ], con
   // where a longer segment lost 20 % on one).  Contiguous rows, two on a unit: a whole segment is
   // what a work-group gets.
   const bool halves = sharing > 2 || (rows_apart && sharing > 1);
-  if (halves) share = 512 / sharing;
-  else if (sharing == 2) share = min(share, 512);
+  if (halves) {
+    // two segments per work-group, 2 * sharing per unit -- unless the unit's load is small: every segment
+    // costs a merge, a store and a restart of the stream whatever its length, so a unit is given one
+    // segment per kSegmentBytesWorthCutting of K and V at most (upstream's own perf shape, 64 sequences of
+    // 1500 keys in byte caches with head size 64: 0.4 MB per unit, and the rows are best left whole)
+    const float load_bytes = items * per_unit * (float)partition_bytes;
+    const int n = max(1, min((int)(load_bytes * (1.0f / (float)kSegmentBytesWorthCutting) + 0.5f), 2 * sharing));
+    share = 1024 / n;
+  } else if (sharing == 2) share = min(share, 512);
   int m = (int)fminf(items * per_unit * ((float)share * (1.0f / 1024.f)) + 0.5f, (float)kSegmentMaxPartitions);
   m = max(m, 1);
   if (m == 1 && items <= (float)groups) return 1;  // a partition per work-group at most: nothing to weigh

@@ -54,7 +54,8 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
              partition_size: int = 0, timed: bool = True, apply_alibi: bool = False,
              apply_softcap: bool = False, window_left: Optional[int] = None,
              k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None,
-             static_scratch_partitions: int = 0, schedule: int = 0, spin_limit: int = 0) -> List[float]:
+             static_scratch_partitions: int = 0, schedule: int = 0, spin_limit: int = 0,
+             segment_partitions: int = 0) -> List[float]:
     """``static_scratch_partitions`` > 0 (split entries without FP8 only): the scratch arrays are the
     library's own fixed device array instead of max_logits / exp_sums / tem_output, which may then be
     None; the value is max_num_partitions."""
@@ -139,6 +140,7 @@ def run_impl(entry: str, split: bool, fp8: bool, max_logits, exp_sums, tem_outpu
     op.query_len = QL
     op.schedule = int(schedule)
     op.spin_limit = int(spin_limit)
+    op.segment_partitions = int(segment_partitions)
     if k_scales is not None or v_scales is not None:
         if not fp8:
             raise _cabi.PagedAttentionError(_cabi.FA_ERR_UNSUPPORTED_DTYPE, "k_scales / v_scales belong to FP8 caches")

@@ -51,7 +51,8 @@ def alloc_buffers(w: Workload, max_num_partitions: Optional[int] = None, fill: f
 def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
                  key_cache: Optional[torch.Tensor] = None,
                  value_cache: Optional[torch.Tensor] = None, timed: bool = True,
-                 max_context_len: Optional[int] = None, schedule: int = 0, spin_limit: int = 0) -> List[float]:
+                 max_context_len: Optional[int] = None, schedule: int = 0, spin_limit: int = 0,
+                 segment_partitions: int = 0) -> List[float]:
     """One call of ``lib.paged_attention_<kernel>.run``; returns its kernel times (us).
     ``key_cache``/``value_cache`` substitute pool clones of the same layout.  ``max_context_len``
     defaults to what the block table can hold (no device read needed to know it).  ``schedule``:
@@ -71,6 +72,7 @@ def run_workload(w: Workload, kernel: str, bufs: Optional[Buffers] = None, *,
     kw = dict(timed=timed, schedule=schedule, spin_limit=spin_limit)
     if "reduce" in kernel:
         kw["partition_size"] = w.partition_size
+        kw["segment_partitions"] = segment_partitions
     if w.is_fp8:
         return mod.run(*head, w.fp8_scale, *tail, **kw)
     return mod.run(*head, *tail, **kw)

@@ -183,6 +183,10 @@ typedef struct fa_paged_attention_options {
                                  void, see fa_paged_attention_kernel_status).  0 = the library's bound,
                                  which no correct run reaches; negative = do not wait at all, which makes
                                  the give-up path run for a test while every kernel still ends normally */
+  int32_t segment_partitions; /* reduce entries, FA_SCHEDULE_AUTO: partitions that one partial covers where
+                                 the library would choose that number itself (see fa_paged_attention_reduce);
+                                 0 = the library chooses, n >= 1 = n (at most 64).  A tuning and test knob:
+                                 `out` does not depend on it beyond the order of fp32 sums */
 } fa_paged_attention_options;
 #define FA_PAGED_ATTENTION_OPTIONS_INIT {(uint32_t)sizeof(fa_paged_attention_options)}
 
@@ -251,6 +255,36 @@ int32_t fa_paged_attention_fp8_reduce(void *out, const void *query, const void *
 
 /* Text of the last failure on the calling thread ("" if none). */
 const char *fa_last_error(void);
+
+/* Which kernels fa_paged_attention_reduce / fa_paged_attention_fp8_reduce (kv_fp8 non-zero) run for a
+ * call of this shape, options and max_context_len -- decided on the host, from these arguments alone:
+ *   FA_SPLIT_FORM_GRID     upstream's decomposition: one work-group and one partial per (sequence, kv
+ *                          head, partition), then the reduce kernel (launch_kernels_reduce.h:18-78)
+ *   FA_SPLIT_FORM_SEGMENT  resident work-groups, one partial per segment of several partitions, then
+ *                          the reduce kernel
+ *   FA_SPLIT_FORM_LOOP     the rows are too short for splitting to pay -- at most 1024 keys, or at most
+ *                          2048 with a (sequence, kv head) row for every compute unit, by what
+ *                          max_context_len (0 = unknown), the block table's width and the scratch
+ *                          arrays' capacity say: the call is the single-pass kernel, one launch; the
+ *                          scratch arrays stay untouched and the second kernel time is 0
+ * compute_units > 0: of the GPU in question; the plan is then made without a device and work_groups
+ * stays 0.  compute_units = 0: the current device's, and work_groups is filled in.  Launches nothing.
+ * No counterpart upstream, whose launcher has one form. */
+typedef enum fa_split_form { FA_SPLIT_FORM_GRID = 0, FA_SPLIT_FORM_SEGMENT = 1, FA_SPLIT_FORM_LOOP = 2 } fa_split_form;
+typedef struct fa_split_plan {
+  uint32_t struct_size;      /* sizeof(fa_split_plan) in the caller's header */
+  int32_t form;              /* fa_split_form */
+  int32_t compute_units;     /* as given, or of the current device */
+  int32_t work_groups;       /* FA_SPLIT_FORM_SEGMENT, made with a device: work-groups of the attention
+                                launch (the first, if the batch takes several); else 0 */
+  int32_t kv_heads_per_item; /* FA_SPLIT_FORM_SEGMENT, made with a device: kv heads that one work item of the
+                                attention kernel covers -- 2 where adjacent heads are taken as pairs or by
+                                teams of wavefronts, else 1; 0 when not filled in */
+} fa_split_plan;
+#define FA_SPLIT_PLAN_INIT {(uint32_t)sizeof(fa_split_plan)}
+int32_t fa_paged_attention_reduce_plan(const fa_paged_attention_shape *shape,
+                                       const fa_paged_attention_options *options, int32_t max_context_len,
+                                       int32_t kv_fp8, int32_t compute_units, fa_split_plan *plan);
 
 /* Did a persistent kernel of the current GPU give up a wait for the wavefronts of its work-group
  * (options->spin_limit) since the word was last cleared?  Then the output of that call is not

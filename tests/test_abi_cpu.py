@@ -40,17 +40,19 @@ def test_struct_layouts_match_header():
     assert _cabi.Shape.kv_block_stride.offset == 40
     assert _cabi.Shape.num_pool_blocks.offset == 68
     assert _cabi.Options.struct_size.offset == 0 and _cabi.Options.sinks.offset == 8
-    assert ctypes.sizeof(_cabi.Options) == 96
+    assert ctypes.sizeof(_cabi.Options) == 104
     assert _cabi.Options.schedule.offset == 88 and _cabi.Options.spin_limit.offset == 92
+    assert _cabi.Options.segment_partitions.offset == 96
     assert _cabi.Options.kv_scale_mode.offset == 68
     assert _cabi.Options.k_scales.offset == 72 and _cabi.Options.v_scales.offset == 80
     assert _cabi.Options.query_len.offset == 64
     assert _cabi.Options.mask_flags.offset == 56 and _cabi.Options.window_left.offset == 60
     assert _cabi.Options.elapsed_us.offset == 40
+    assert ctypes.sizeof(_cabi.SplitPlan) == 20 and _cabi.SplitPlan.kv_heads_per_item.offset == 16
     assert ctypes.sizeof(_cabi.KvWriteShape) == 4 + 4 * 4 + 4 + 5 * 8 + 2 * 4 + 8 == 80
     assert _cabi.KvWriteShape.src_dtype.offset == 64 and _cabi.KvWriteShape.num_pool_blocks.offset == 72
     # a new struct says how large it is
-    assert _cabi.Shape().struct_size == 72 and _cabi.Options().struct_size == 96 and _cabi.KvWriteShape().struct_size == 80
+    assert _cabi.Shape().struct_size == 72 and _cabi.Options().struct_size == 104 and _cabi.KvWriteShape().struct_size == 80
 
 
 def test_header_struct_sizes_agree_with_the_compiler(tmp_path):
@@ -72,7 +74,7 @@ def test_header_struct_sizes_agree_with_the_compiler(tmp_path):
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
                    check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert [int(x) for x in out] == [72, 96, 80, 68, 88, 92, 72, 0]
+    assert [int(x) for x in out] == [72, 104, 80, 68, 88, 92, 72, 0]
 
 
 def test_shorter_and_longer_structs(L):
@@ -106,7 +108,7 @@ def test_shorter_and_longer_structs(L):
     assert call(options_size=_cabi.Options.spin_limit.offset, schedule=3)[0] == _cabi.FA_ERR_BAD_SHAPE
     # the shortest struct this test may pass ends with validate_only (without it the call would launch)
     assert call(options_size=_cabi.Options.validate_only.offset + 4, schedule=3) == (_cabi.FA_OK, "")
-    for bad in (0, 2, 97, 100, 1 << 20):
+    for bad in (0, 2, 97, 108, 1 << 20):
         rc, msg = call(options_size=bad)
         assert rc == _cabi.FA_ERR_BAD_SHAPE and "options.struct_size" in msg, (bad, msg)
     for bad in (0, 36, 68, 70, 76, 4096):  # every field of the shape is needed
