@@ -63,17 +63,37 @@ HBM_PEAK_GBPS = 8000.0
 # 512-sequence variants of the configurations (--large-batches): blocks per pool
 LARGE_BATCH_POOL_BLOCKS = {1: 49152, 3: 49152, 4: 220000}
 
+def kernel_sources_digest():
+    """sha256 over the kernel sources (csrc/*.h, csrc/*.hip, names and contents in sorted order): what
+    ties a counter measurement to the code it was made on."""
+    import hashlib
+    h = hashlib.sha256()
+    folder = os.path.join(ROOT, "flash_attention_factory_amd", "csrc")
+    for name in sorted(os.listdir(folder)):
+        if name.endswith((".h", ".hip")):
+            h.update(name.encode())
+            h.update(open(os.path.join(folder, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
 def _measured_traffic():
     """HBM bytes per launch of each configuration's dominant kernel, from the rocprofv3 --pmc
     FETCH_SIZE / WRITE_SIZE runs summarised in profiles/hbm_traffic.txt (lines: name fetch_MB
-    write_MB).  None for a configuration the file does not list."""
+    write_MB).  The file names the digest of the kernel sources it was measured on ("# csrc:"); if
+    the sources have changed since, nothing is reported (None), and None for a configuration the
+    file does not list."""
     table = {}
     path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     if os.path.exists(path):
+        measured_on = None
         for line in open(path):
             parts = line.split()
-            if len(parts) >= 3 and not line.startswith("#"):
+            if line.startswith("# csrc:") and len(parts) >= 3:
+                measured_on = parts[2]
+            elif len(parts) >= 3 and not line.startswith("#"):
                 table[parts[0]] = (float(parts[1]) + float(parts[2])) * 1e6
+        if measured_on != kernel_sources_digest():
+            return {}
     return table
 
 
@@ -262,17 +282,28 @@ def _reference_perf_recipe(steps, torch, W, runner, dev):
         w.meta["kernel"] = "fp8_loop" if fp8 else "loop"
         pool_bytes = w.key_cache.numel() * w.key_cache.element_size() * 2
         ks, vs = _clones(w, torch)
-        for kernel in ((("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce"))):
+        pre = "fp8_" if fp8 else ""
+        # loop entry; split entry as upstream calls it; split entry made to run its two kernels (whole rows
+        # as one segment each, and upstream's one partial per partition)
+        for kernel, forced in ((pre + "loop", {}), (pre + "reduce", {}), (pre + "reduce", dict(segment_partitions=64)),
+                               (pre + "reduce", dict(schedule=1))):
             bufs = runner.alloc_buffers(w)
             ts = []
             for it in range(5 + steps):
-                t = runner.run_workload(w, kernel, bufs, key_cache=ks[it % len(ks)], value_cache=vs[it % len(ks)])
+                # upstream passes seqlen_k as max_context_len (test_paged.py:478-480)
+                t = runner.run_workload(w, kernel, bufs, key_cache=ks[it % len(ks)], value_cache=vs[it % len(ks)],
+                                        max_context_len=1500, **forced)
                 if it >= 5:
                     ts.append(sum(t))
             us = float(torch.tensor(ts, dtype=torch.float64).mean())
+            form = None
+            if "reduce" in kernel:  # which kernels the split entry ran
+                form = "single-pass kernel" if t[1] == 0.0 else "split kernels"
+                if forced:
+                    form += " (forced: " + ", ".join(f"{k}={v}" for k, v in forced.items()) + ")"
             legs.append(dict(workload=f"upstream perf recipe: S64 H{heads} Hk8 D64 B64 ctx1500 sinks, token-major, "
                                       f"{'E5M2' if fp8 else 'fp16'} pools", kernel=kernel, steps=steps,
-                             us_per_call=us, pool_clones=len(ks), whole_pool_bytes=pool_bytes,
+                             us_per_call=us, form=form, pool_clones=len(ks), whole_pool_bytes=pool_bytes,
                              gbps_whole_pool=pool_bytes / us / 1e3,
                              algorithmic_bytes=w.algorithmic_bytes(), gbps_kernels=w.algorithmic_bytes() / us / 1e3,
                              hbm_frac=w.algorithmic_bytes() / us / 1e3 / HBM_PEAK_GBPS))
@@ -517,14 +548,30 @@ def main():
                     help="also time configurations 4, 3 and 1 with 512 sequences (up to 26 GB of pools), "
                          "each in a process of its own")
     ap.add_argument("--large-batch-only", type=int, default=-1, help=argparse.SUPPRESS)
+    ap.add_argument("--calibrate-counters", action="store_true",
+                    help="run nothing but three plain device-to-device copies of 1 GiB (read 1 GiB, write 1 GiB "
+                         "each): under rocprofv3 --pmc FETCH_SIZE or WRITE_SIZE their readings give the scale of "
+                         "the counter")
+    ap.add_argument("--sources-digest", action="store_true", help="print the digest of the kernel sources and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no multi-GPU form in this build "
               f"(--gpus {args.gpus} refused)", file=sys.stderr)
         return 2
 
+    if args.sources_digest:
+        print(kernel_sources_digest())
+        return 0
     import torch
     from flash_attention_factory_amd import _cabi, runner, workloads as W
+    if args.calibrate_counters:
+        src = torch.full((1 << 30,), 0x5a, dtype=torch.uint8, device="cuda:0")
+        dst = torch.zeros_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "3 device-to-device copies", "read_bytes_each": 1 << 30, "written_bytes_each": 1 << 30}))
+        return 0
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
@@ -646,8 +693,29 @@ def main():
                 print(child.stderr, file=sys.stderr)
                 return child.returncode
             line["large_batches"].append(json.loads(child.stdout.strip().splitlines()[-1]))
+    # Every configuration's figures once more, compact and LAST in the line (and inside `config`), so
+    # that whoever keeps only the head or the tail of it keeps them: microseconds per call, the dominant
+    # kernel's duration and fraction of the HBM peak, measured traffic.
+    summary = [_summary_of("config1: " + args.layout, main_res["us_per_call"], line["roofline"])]
+    for r in others:
+        summary.append(_summary_of(r["workload"], r["us_per_call"], r["roofline"], r.get("kernel_us_mean")))
+    for r in line.get("reference_perf_recipe", []):
+        if r.get("form") is None or "forced" not in r["form"]:
+            summary.append(dict(w=("recipe_e5m2_" if "E5M2" in r["workload"] else "recipe_fp16_") + r["kernel"],
+                                us=round(r["us_per_call"], 2), frac=round(r["hbm_frac"], 4), form=r.get("form")))
+    line["config"]["configs_summary"] = summary
+    line["configs_summary"] = summary
     print(json.dumps(line), flush=True)
     return 0
+
+
+def _summary_of(name, us_per_call, roofline, kernel_us_mean=None):
+    out = dict(w=name, us=round(us_per_call, 2), kernel_us=round(roofline["kernel_us"], 2),
+               GBps=round(roofline["achieved"], 1), frac=round(roofline["frac"], 4),
+               traffic_MB=None if roofline["traffic"] is None else round(roofline["traffic"] / 1e6, 2))
+    if kernel_us_mean and len(kernel_us_mean) > 1:
+        out["reduce_us"] = round(kernel_us_mean[1], 2)
+    return out
 
 
 if __name__ == "__main__":

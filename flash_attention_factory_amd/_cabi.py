@@ -56,6 +56,7 @@ FA_KV_SCALE_BLOCK = 2
 FA_SCHEDULE_AUTO = 0
 FA_SCHEDULE_GRID = 1
 FA_SCHEDULE_GRID_LDS = 2
+FA_SCHEDULE_SPLIT = 3
 
 FA_SPLIT_FORM_GRID = 0
 FA_SPLIT_FORM_SEGMENT = 1

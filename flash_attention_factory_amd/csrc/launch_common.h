@@ -152,7 +152,8 @@ struct Resolved {
   int32_t kv_scale_mode;  // fa_kv_scale; with a mode other than 0 fp8_scale is 1
   const float *k_scales;
   const float *v_scales;
-  int32_t schedule;  // fa_schedule
+  int32_t schedule;  // fa_schedule (FA_SCHEDULE_SPLIT: FA_SCHEDULE_AUTO with keep_split)
+  bool keep_split;   // a reduce entry runs its two kernels however short the rows
   int32_t segment_partitions;  // > 0: partitions per partial of the segment form, fixed by the caller
   bool pair_heads;   // two adjacent kv heads with 64-byte token rows run as one (WaveAttn::kPairable)
   int32_t *status;   // status word of the current device (nullptr with validate_only)
@@ -262,8 +263,12 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
     r->fp8_scale = 1.0f;
   }
   r->schedule = o ? o->schedule : FA_SCHEDULE_AUTO;
-  if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS)
-    return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2)", r->schedule);
+  if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS &&
+      r->schedule != FA_SCHEDULE_SPLIT)
+    return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2), split (3)",
+                r->schedule);
+  r->keep_split = r->schedule == FA_SCHEDULE_SPLIT;  // otherwise the library's own choice
+  if (r->keep_split) r->schedule = FA_SCHEDULE_AUTO;
   r->segment_partitions = o ? o->segment_partitions : 0;
   if (r->segment_partitions < 0) return fail(FA_ERR_BAD_SHAPE, "segment_partitions must be >= 0");
   r->pair_heads = kPairHeads && kv8 && s->head_size == 64 && s->kv_head_stride == s->head_size &&

@@ -69,7 +69,7 @@ inline SplitForm split_form_of(const fa_paged_attention_shape &shape, const Reso
                                int32_t max_context_len, int compute_units) {
   if (r.schedule != FA_SCHEDULE_AUTO) return kSplitFormGrid;
   const bool loop_persistent = loop_persistent_fits(shape) && shape.num_seqs <= kLoopPersistentMaxSeqs;
-  if (loop_persistent && r.segment_partitions == 0 &&
+  if (loop_persistent && r.segment_partitions == 0 && !r.keep_split &&
       split_call_runs_as_loop(split_row_bound(shape, r.partition_size, max_context_len), loop_rows_of(shape, r, kv8),
                               compute_units))
     return kSplitFormLoop;

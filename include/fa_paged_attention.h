@@ -113,8 +113,13 @@ typedef enum fa_mask { FA_MASK_ALIBI = 1, FA_MASK_SOFTCAP = 2, FA_MASK_WINDOW = 
  * paged_attention_kernel_v2.hpp:562-569): every live slot of exp_sums / max_logits / tmp_out then
  * holds exactly what upstream stores there.  FA_SCHEDULE_GRID_LDS is the grid form with K and V
  * staged through LDS by direct-to-LDS loads (FP8 entries, head size 128, no score modifiers;
- * anything else falls back to FA_SCHEDULE_GRID).  `out` is the same under all three. */
-typedef enum fa_schedule { FA_SCHEDULE_AUTO = 0, FA_SCHEDULE_GRID = 1, FA_SCHEDULE_GRID_LDS = 2 } fa_schedule;
+ * anything else falls back to FA_SCHEDULE_GRID).  FA_SCHEDULE_SPLIT is FA_SCHEDULE_AUTO except that a
+ * reduce entry always runs its two kernels, also where rows are so short that FA_SCHEDULE_AUTO runs the
+ * single-pass kernel instead (fa_paged_attention_reduce_plan); loop entries take it as FA_SCHEDULE_AUTO.
+ * `out` is the same under all four. */
+typedef enum fa_schedule {
+  FA_SCHEDULE_AUTO = 0, FA_SCHEDULE_GRID = 1, FA_SCHEDULE_GRID_LDS = 2, FA_SCHEDULE_SPLIT = 3
+} fa_schedule;
 
 typedef enum fa_kv_scale { FA_KV_SCALE_TENSOR = 0, FA_KV_SCALE_HEAD = 1, FA_KV_SCALE_BLOCK = 2 } fa_kv_scale;
 

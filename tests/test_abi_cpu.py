@@ -102,12 +102,12 @@ def test_shorter_and_longer_structs(L):
         return L.fa_paged_attention_loop(p, p, p, p, p, p, 0.1, 0, ctypes.byref(sh), ctypes.byref(op)), L.fa_last_error().decode()
 
     assert call() == (_cabi.FA_OK, "")
-    assert call(schedule=3)[0] == _cabi.FA_ERR_BAD_SHAPE                      # the field is read ...
+    assert call(schedule=9)[0] == _cabi.FA_ERR_BAD_SHAPE                      # the field is read ...
     before_schedule = _cabi.Options.schedule.offset
-    assert call(options_size=before_schedule, schedule=3) == (_cabi.FA_OK, "")  # ... unless the caller's struct ends before it
-    assert call(options_size=_cabi.Options.spin_limit.offset, schedule=3)[0] == _cabi.FA_ERR_BAD_SHAPE
+    assert call(options_size=before_schedule, schedule=9) == (_cabi.FA_OK, "")  # ... unless the caller's struct ends before it
+    assert call(options_size=_cabi.Options.spin_limit.offset, schedule=9)[0] == _cabi.FA_ERR_BAD_SHAPE
     # the shortest struct this test may pass ends with validate_only (without it the call would launch)
-    assert call(options_size=_cabi.Options.validate_only.offset + 4, schedule=3) == (_cabi.FA_OK, "")
+    assert call(options_size=_cabi.Options.validate_only.offset + 4, schedule=9) == (_cabi.FA_OK, "")
     for bad in (0, 2, 97, 108, 1 << 20):
         rc, msg = call(options_size=bad)
         assert rc == _cabi.FA_ERR_BAD_SHAPE and "options.struct_size" in msg, (bad, msg)
@@ -311,9 +311,9 @@ def test_kv_scale_argument_checks(L):
 def test_schedule_values(L):
     for split in (False, True):
         for fp8 in (False, True):
-            for schedule in (0, 1, 2):  # the LDS form falls back to the grid form where it does not apply
+            for schedule in (0, 1, 2, 3):  # the LDS form falls back to the grid form where it does not apply
                 assert _call(L, split=split, fp8=fp8, schedule=schedule)[0] == _cabi.FA_OK
-            code, text = _call(L, split=split, fp8=fp8, schedule=3)
+            code, text = _call(L, split=split, fp8=fp8, schedule=4)
             assert code == _cabi.FA_ERR_BAD_SHAPE and "schedule" in text
 
 

@@ -23,12 +23,18 @@ def _dev():
     return torch.device("cuda:0")
 
 
-def _run(w_cpu, kernel, max_context_len=None, schedule=0, spin_limit=0, timed=True, **kw):
+def _run(w_cpu, kernel, max_context_len=None, schedule=0, spin_limit=0, timed=True, segment_partitions=0, **kw):
     from flash_attention_factory_amd import runner
     w = w_cpu.to(_dev())
     bufs = runner.alloc_buffers(w, **kw)
     times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len, schedule=schedule,
-                                spin_limit=spin_limit, timed=timed)
+                                spin_limit=spin_limit, timed=timed, segment_partitions=segment_partitions)
+    if "reduce" in kernel and timed and times[1] == 0.0:
+        # rows so short that the split entry ran the single-pass kernel (tests/test_gpu_segment_policy.py
+        # covers that); the tests here are after the split kernels
+        bufs = runner.alloc_buffers(w, **kw)
+        times = runner.run_workload(w, kernel, bufs, max_context_len=max_context_len, schedule=3,
+                                    spin_limit=spin_limit)
     torch.cuda.synchronize()
     return bufs, times
 
@@ -449,7 +455,7 @@ def test_full_size_configs(oracle, index, layout):
     _check(bufs.out, w, oracle, f"full {w.name}, {layout}")
     other = {"loop": "reduce", "reduce": "loop", "fp8_loop": "fp8_reduce", "fp8_reduce": "fp8_loop"}[kernel]
     bufs2 = runner.alloc_buffers(wd)
-    runner.run_workload(wd, other, bufs2)
+    runner.run_workload(wd, other, bufs2, schedule=3)  # the split kernels also where the rows are short
     torch.cuda.synchronize()
     a, b = bufs.out.float(), bufs2.out.float()
     ulps = 2.0 ** (-7 if w.query.dtype == torch.bfloat16 else -10)  # two 16-bit roundings apart
@@ -662,9 +668,11 @@ def test_whole_upstream_grid(oracle, heads, fp8):
     absolute one, twice: err <= 3 x err of the rounding-faithful kernel model + 1e-5, and literally,
     err <= 3 x err(out_pt) + 1e-5 with out_pt the reference evaluated without the fp32 upcast
     (test_paged.py:432-447, 603-604).
-    The seven lengths up to 2048 in full; of the three long ones (20000-50000) one combination of
-    the other parameters each, rotating -- the oracle needs a third of a second for those -- unless
-    FA_FULL_UPSTREAM_GRID=1 asks for all 2 x 1440 cases."""
+    All 2 x 1440 cases (two minutes, most of it the oracle on the three long lengths); with
+    FA_QUICK_UPSTREAM_GRID=1 the seven lengths up to 2048 in full and of the long ones (20000-50000)
+    one combination of the other parameters each, rotating.  (Rows of up to 1024 keys would make the
+    split entry run the single-pass kernel, which the loop entry covers: _run asks for the split
+    kernels there.)"""
     nheads, nheads_k = heads
     combos = [(b, s, v, d) for b in (1, 2) for s in (True, False) for v in (False, True) for d in (128, 64)]
     n = 0
@@ -673,10 +681,11 @@ def test_whole_upstream_grid(oracle, heads, fp8):
             w = W.make_test_shaped(batch_size=b, nheads=nheads, nheads_k=nheads_k, d=d, seqlen_k=seqlen_k, varlen=v,
                                    has_sinks=s, fp8=fp8)
             for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
-                bufs, _ = _run(w, kernel)
+                bufs, times = _run(w, kernel)  # (the split kernels also where rows are short: see _run)
+                assert "reduce" not in kernel or times[1] > 0.0
                 _check(bufs.out, w, oracle, f"{w.name}/{kernel}", literal_rule=True)
             n += 1
-    everything = os.environ.get("FA_FULL_UPSTREAM_GRID") == "1"   # the long lengths in full too: minutes
+    everything = os.environ.get("FA_QUICK_UPSTREAM_GRID") != "1"   # the long lengths in full too
     for k, seqlen_k in enumerate(UPSTREAM_LONG):
         one = combos[(3 * UPSTREAM_HEADS.index(heads) + k + (8 if fp8 else 0)) % len(combos)]
         for b, s, v, d in (combos if everything else [one]):

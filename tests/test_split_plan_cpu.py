@@ -57,6 +57,7 @@ def test_upstreams_perf_shapes_run_as_the_single_pass_kernel(L):
     # a caller who asks for upstream's decomposition, or fixes the segment length, gets the split kernels
     assert _plan(L, H=64, max_context_len=1500, schedule=_cabi.FA_SCHEDULE_GRID, **recipe) == GRID
     assert _plan(L, H=64, max_context_len=1500, segment_partitions=2, **recipe) == SEGMENT
+    assert _plan(L, H=64, max_context_len=1500, schedule=_cabi.FA_SCHEDULE_SPLIT, **recipe) == SEGMENT
 
 
 def test_benchmark_configurations(L):
