@@ -203,6 +203,22 @@ FA_EXPORT int32_t fa_paged_attention_kernel_status(void *stream, int32_t clear) 
   return fa::read_kernel_status(reinterpret_cast<hipStream_t>(stream), clear != 0, 0);
 }
 
+#ifdef FA_TIMELINE
+// Debug builds only (-DFA_TIMELINE): the in-kernel timeline of the current device, copied to the host
+// (kTimelineWaves x kTimelineSlots 64-bit words), and cleared on request.
+FA_EXPORT int32_t fa_debug_timeline(void *dst, size_t bytes, int32_t clear) {
+  const size_t all = sizeof(unsigned long long) * fa::kTimelineWaves * fa::kTimelineSlots;
+  FA_HIP_CHECK(hipDeviceSynchronize());
+  FA_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(fa::timeline_words), bytes < all ? bytes : all));
+  if (clear) {
+    void *address = nullptr;
+    FA_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(fa::timeline_words)));
+    FA_HIP_CHECK(hipMemset(address, 0, all));
+  }
+  return FA_OK;
+}
+#endif
+
 FA_EXPORT const char *fa_last_error(void) { return fa::error_buffer(); }
 
 FA_EXPORT int32_t fa_paged_attention_abi_version(void) { return fa::kAbiRevision; }

@@ -154,7 +154,7 @@ struct Resolved {
   const float *v_scales;
   int32_t schedule;  // fa_schedule (FA_SCHEDULE_SPLIT: FA_SCHEDULE_AUTO with keep_split)
   bool keep_split;   // a reduce entry runs its two kernels however short the rows
-  int32_t segment_partitions;  // > 0: partitions per partial of the segment form, fixed by the caller
+  int32_t segment_partitions;  // > 0: partitions per partial of the segment form, fixed by the caller; -1: even shares
   bool pair_heads;   // two adjacent kv heads with 64-byte token rows run as one (WaveAttn::kPairable)
   int32_t *status;   // status word of the current device (nullptr with validate_only)
   int32_t spin_limit;
@@ -270,7 +270,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   r->keep_split = r->schedule == FA_SCHEDULE_SPLIT;  // otherwise the library's own choice
   if (r->keep_split) r->schedule = FA_SCHEDULE_AUTO;
   r->segment_partitions = o ? o->segment_partitions : 0;
-  if (r->segment_partitions < 0) return fail(FA_ERR_BAD_SHAPE, "segment_partitions must be >= 0");
+  if (r->segment_partitions < -2)
+    return fail(FA_ERR_BAD_SHAPE, "segment_partitions must be -2 (segments of the library's length), -1 (even shares), "
+                                  "0 (the library chooses) or a count");
   r->pair_heads = kPairHeads && kv8 && s->head_size == 64 && s->kv_head_stride == s->head_size &&
                   s->num_kv_heads % 2 == 0 && 2 * r->group <= kMaxGroup && r->mask_flags == 0 &&
                   r->query_len == 1 && r->kv_scale_mode == FA_KV_SCALE_TENSOR;

@@ -3,10 +3,12 @@
 // of this work-group.  Two lists, one interface:
 //
 //   LoopItems     loop path: one item per (sequence, kv head), sequences longest first.
-//   SegmentItems  split path: one item per (sequence, kv head, segment of m partitions), all
-//                 full segments first, then the sequences' last, shorter segments by length
-//                 (what paged_attention_segment_kernel.h deals, and what the reduce kernel
-//                 expects: one partial per segment, in the slot of its first partition).
+//   SegmentItems  split path, one item per piece of a (sequence, kv head) row.  Either segments of m
+//                 partitions -- all full segments first, then the sequences' last, shorter
+//                 segments by length -- or even shares: the rows' partitions laid end to end
+//                 (sequences in order, kv heads within a sequence) and cut into one contiguous share
+//                 per work-group (paged_attention_segment_policy.h).  One partial per piece, in the
+//                 slot of its first partition.
 //
 // Both deal the sorted list to the work-groups in snake order: work-group j takes positions
 // j, 2G-1-j, 2G+j, ... so that a handful of items per work-group still add up evenly.
@@ -18,8 +20,9 @@
 namespace fa {
 
 // chunks c_lo .. c_end-1 of CT tokens; tok_end: where the item's keys end (the context's end, or
-// the segment's); part0: slot of the item's partial (split path); ctx: the sequence's length
-struct WorkItem { int seq, kvh, ctx, c_lo, c_end, tok_end, part0; };
+// the piece's); part0: slot of the item's partial and parts: partitions it covers (split path);
+// ctx: the sequence's length
+struct WorkItem { int seq, kvh, ctx, c_lo, c_end, tok_end, part0, parts; };
 
 __device__ __forceinline__ int snake_position(int nth, int groups, int group) {
   return nth * groups + ((nth & 1) ? groups - 1 - group : group);
@@ -99,6 +102,7 @@ struct LoopItems {
     it.c_lo = 0;
     it.c_end = (it.ctx + chunk_tokens - 1) / chunk_tokens;
     it.part0 = 0;
+    it.parts = 1;
     return it.ctx > 0;  // sorted: nothing but empty sequences follows an empty one
   }
   // block id of tile t of chunk `wave` of a sequence, as requested with the lengths
@@ -109,8 +113,13 @@ struct LoopItems {
 
 struct SegmentItems {
   static constexpr int NQ = kSegmentMaxSeqs / 64;
-  int ctxv[NQ], parts[NQ], incl[NQ], fullc[NQ], key[NQ], rank[NQ];
-  int S, Hk, m, seg_tokens, full_total, total_items, lane;
+  int ctxv[NQ], parts[NQ], incl[NQ], fullc[NQ], key[NQ];
+  int S, Hk, m, seg_tokens, full_total, total_items, lane, key_top_bit, psize;
+  // even shares (m == 0): tape[j] = cost of all rows up to and including the lane's sequence's (row_cost);
+  // the work-group's share is [cursor, share_end) of that tape
+  bool even;
+  int tape[NQ], cursor, share_end, steps_per_partition;
+  float inv_steps_per_partition;
 
   // Lane holds sequences lane, lane + 64, ...  m, the partitions per segment, follows from the
   // batch, the number of work-groups and the compute units they share (partitions_per_segment).
@@ -122,7 +131,15 @@ struct SegmentItems {
     S = p.num_seqs;
     Hk = p.num_kv_heads / heads_per_item;
     const int max_ctx = p.max_blocks_per_seq << p.block_shift;
+    psize = p.partition_size;
     const int total_parts = count_partitions<NQ>(p.context_lens, S, max_ctx, p.partition_size, p.max_num_partitions, lane, ctxv, parts);
+    // (cost of the batch in steps of kShareTokens, from above: every partition full, every row a piece)
+    const long long steps_at_most = ((long long)total_parts * (psize >> kShareTokensLog2) + (long long)S * kSharePieceCost) * Hk;
+    even = p.segment_force == -1 && steps_at_most < (1 << 24);  // (a batch beyond that is cut into segments)
+    if (even) {
+      build_even_shares(groups, p.compute_units);
+      return;
+    }
     m = p.segment_force > 0 ? min(p.segment_force, kSegmentMaxPartitions)
                             : partitions_per_segment<NQ>(ctxv, parts, total_parts, S, p.partition_size, Hk, groups,
                                                          p.compute_units, p.kv_rows_apart != 0,
@@ -135,40 +152,136 @@ struct SegmentItems {
       ctxv[j] = cut;
       fullc[j] = cut / seg_tokens;
       const int rem = cut - fullc[j] * seg_tokens;
-      // sort key of the last segment: length, then lower sequence number first; -1: none
-      key[j] = rem > 0 ? (rem << 8) | (255 - (lane + 64 * j)) : -1;
-      rank[j] = 0;
+      // sort key of the last segment: length in 32-token steps (what a wavefront takes at a time),
+      // then lower sequence number first; -1: none
+      key[j] = rem > 0 ? (((rem + 31) >> 5) << 8) | (255 - (lane + 64 * j)) : -1;
       int x = fullc[j];
       if (j * 64 < S) {
         tails += __builtin_popcountll(__ballot(rem > 0));
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-          const int y = __shfl_up(x, o);
-          if (lane >= o) x += y;
-        }
+        x = wave_inclusive_sum(x);
       }
       incl[j] = x + running;
       running = __builtin_amdgcn_readlane(incl[j], 63);
     }
     full_total = running;
     total_items = (full_total + tails) * Hk;
-    // rank of every last segment among the last segments (how many are longer)
+    // highest pair of bits a key can have: lengths of last segments stay below seg_tokens
+    key_top_bit = (31 - __builtin_clz(((unsigned)((min(seg_tokens, kSegmentMaxContext - 1) + 31) >> 5) << 8) | 255u)) & ~1;
+  }
+  // Even shares.  A row costs its keys in steps of kShareTokens plus kSharePieceCost steps for what
+  // every piece costs whatever its length (a merge, a store, a start without loads in flight).  The
+  // rows' costs lie end to end on a tape; a work-group's share is a contiguous stretch of it.
+  __device__ __forceinline__ int row_cost(int ctx) const {
+    return ctx > 0 ? ((ctx + kShareTokens - 1) >> kShareTokensLog2) + kSharePieceCost : 0;
+  }
+  __device__ __forceinline__ void build_even_shares(int groups, int cus) {
+    m = 0;
+    seg_tokens = 0;
+    int running = 0;
 #pragma unroll
-    for (int js = 0; js < NQ; ++js) {
-      if (js * 64 < S) {
-        for (int u0 = 0; u0 < min(S - js * 64, 64); u0 += 8) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int ku = __builtin_amdgcn_readlane(key[js], u0 + e);
-#pragma unroll
-            for (int jd = 0; jd < NQ; ++jd) rank[jd] += ku > key[jd];
-          }
-        }
+    for (int j = 0; j < NQ; ++j) {
+      ctxv[j] = min(ctxv[j], parts[j] * psize);  // what the scratch arrays can hold
+      int x = row_cost(ctxv[j]);
+      if (j * 64 < S) x = wave_inclusive_sum(x);
+      tape[j] = (x + running) * Hk;
+      running = __builtin_amdgcn_readlane(x + running, 63);
+    }
+    const int n = running * Hk;  // below 2^24: SegmentItems::build
+    // Two work-groups on every compute unit (g and g + cus): the hardware serves the older of the two
+    // first, so that with equal shares it is through early and the younger one streams on alone, below
+    // the unit's rate.  The older half of the work-groups takes kShareOlderPermille of the tape, so
+    // that both are through together.
+    int count = groups, g = (int)blockIdx.x, begin = 0, length = n;
+    if (groups == 2 * cus) {
+      const int older = (int)((float)n * (kShareOlderPermille * 0.001f));
+      count = cus;
+      if (g >= cus) {
+        g -= cus;
+        begin = older;
+        length = n - older;
+      } else {
+        length = older;
       }
     }
+    int extra;
+    const int each = quotient_below_2p24(length, count, __builtin_amdgcn_rcpf((float)count), extra);
+    cursor = begin + g * each + min(g, extra);  // the first `extra` work-groups take one step more
+    share_end = cursor + each + (g < extra ? 1 : 0);
+    total_items = n;
+    steps_per_partition = psize >> kShareTokensLog2;
+    inv_steps_per_partition = __builtin_amdgcn_rcpf((float)steps_per_partition);
   }
-  // position in the sorted list -> (sequence, segment, kv head), kv head fastest
-  __device__ __forceinline__ bool at(int n, int groups, int group, int chunk_tokens, WorkItem &it) const {
+  // The partition boundary of a row of `parts` partitions nearest to cost position x of the row: where a
+  // share that ends (or begins) there really ends (begins), since a piece is whole partitions.  Two
+  // neighbouring work-groups evaluate it at the same position of the same row.
+  __device__ __forceinline__ int nearest_cut(int x, int parts_of_row) const {
+    int rem;
+    return min(parts_of_row, quotient_below_2p24(x + (steps_per_partition >> 1), steps_per_partition, inv_steps_per_partition, rem));
+  }
+  // Next piece of this work-group's share: what the share holds of the row the cursor lies in.
+  __device__ __forceinline__ bool next_of_share(int chunk_tokens, WorkItem &it) {
+    while (cursor < share_end) {  // (a row of which rounding leaves the share nothing is passed over)
+      int s = 0;
+#pragma unroll
+      for (int j = 0; j < NQ; ++j)
+        if (j * 64 < S) s += __builtin_popcountll(__ballot(lane + 64 * j < S && tape[j] <= cursor));
+      s = min(s, S - 1);
+      int tape_s = 0, parts_s = 1, ctx_s = 0;
+#pragma unroll
+      for (int j = 0; j < NQ; ++j)
+        if ((s >> 6) == j) {
+          tape_s = __builtin_amdgcn_readlane(tape[j], s & 63);
+          parts_s = __builtin_amdgcn_readlane(parts[j], s & 63);
+          ctx_s = __builtin_amdgcn_readlane(ctxv[j], s & 63);
+        }
+      const int cost = max(row_cost(ctx_s), 1);
+      const int into = cursor - (tape_s - cost * Hk);  // into the sequence's rows: kv head x cost + position in the row
+      int x;
+      const int kvh = quotient_below_2p24(into, cost, __builtin_amdgcn_rcpf((float)cost), x);
+      const int row_begin = cursor - x, row_end = row_begin + cost;
+      const int from = x == 0 ? 0 : nearest_cut(x, parts_s);
+      const int to = share_end >= row_end ? parts_s : nearest_cut(share_end - row_begin, parts_s);
+      cursor = min(row_end, share_end);
+      if (to > from) {
+        it.seq = __builtin_amdgcn_readfirstlane(s);
+        it.kvh = __builtin_amdgcn_readfirstlane(kvh);
+        it.ctx = ctx_s;
+        it.part0 = __builtin_amdgcn_readfirstlane(from);
+        it.parts = __builtin_amdgcn_readfirstlane(to - from);
+        it.tok_end = to == parts_s ? ctx_s : to * psize;
+        it.c_lo = from * psize / chunk_tokens;
+        it.c_end = (it.tok_end + chunk_tokens - 1) / chunk_tokens;
+        return true;
+      }
+    }
+    return false;
+  }
+  // The sequence whose last segment is the rho-th longest (0: the longest).  The keys are distinct, so
+  // the one that exactly rho others exceed is found from the top, two bits at a time (three counts
+  // that do not depend on each other) -- when an item is looked up, one at a time and as a rule
+  // behind loads that are already in flight; ranking all sequences against each other before the
+  // first load cost a launch of 128 sequences 4 to 7 microseconds.
+  __device__ __forceinline__ int sequence_of_tail(int rho) const {
+    int found = 0;
+#pragma nounroll
+    for (int bit = key_top_bit; bit >= 0; bit -= 2) {
+      int at_least[3] = {0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < NQ; ++j)
+        if (j * 64 < S) {
+#pragma unroll
+          for (int c = 0; c < 3; ++c) at_least[c] += __builtin_popcountll(__ballot(key[j] >= (found | ((c + 1) << bit))));
+        }
+      // counts fall with the candidate: the largest one that more than rho keys still reach
+      const int digit = (at_least[0] > rho) + (at_least[1] > rho) + (at_least[2] > rho);
+      found |= digit << bit;
+    }
+    return 255 - (found & 255);
+  }
+  // n-th item of work-group `group`, asked for n = 0, 1, 2, ... in turn.  Segments: position in the
+  // sorted list -> (sequence, segment, kv head), kv head fastest.
+  __device__ __forceinline__ bool at(int n, int groups, int group, int chunk_tokens, WorkItem &it) {
+    if (even) return next_of_share(chunk_tokens, it);
     const int pos = snake_position(n, groups, group);
     if (pos >= total_items) return false;
     const int q = __builtin_amdgcn_readfirstlane(pos / Hk);
@@ -180,13 +293,7 @@ struct SegmentItems {
       for (int j = 0; j < NQ; ++j)
         if (j * 64 < S) s += __builtin_popcountll(__ballot(lane + 64 * j < S && incl[j] <= q));
     } else {
-      const int rho = q - full_total;
-#pragma unroll
-      for (int j = 0; j < NQ; ++j)
-        if (j * 64 < S) {
-          const unsigned long long hit = __ballot(key[j] >= 0 && rank[j] == rho);
-          if (hit) s = 64 * j + __builtin_ctzll(hit);
-        }
+      s = sequence_of_tail(q - full_total);
     }
     s = min(s, S - 1);
     int inc_s = 0, full_s = 0, ctx_s = 0;
@@ -202,6 +309,7 @@ struct SegmentItems {
     it.part0 = seg * m;
     const int tok_begin = seg * seg_tokens;
     it.tok_end = full ? tok_begin + seg_tokens : ctx_s;
+    it.parts = (it.tok_end - tok_begin + psize - 1) / psize;
     it.c_lo = tok_begin / chunk_tokens;
     it.c_end = (it.tok_end + chunk_tokens - 1) / chunk_tokens;
     it.ctx = ctx_s;

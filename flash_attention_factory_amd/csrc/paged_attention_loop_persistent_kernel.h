@@ -25,6 +25,20 @@
 #include "paged_attention_items.h"
 #include "paged_attention_kernel.h"
 
+// (debug builds with -DFA_TIMELINE) after a score pass: count it, and stamp the first one of the wavefront
+#ifdef FA_TIMELINE
+#define FA_TIMELINE_QK()              \
+  do {                                \
+    ++timeline_chunks;                \
+    if (timeline_first) {             \
+      timeline_first = false;         \
+      FA_TIMELINE_STAMP(2);           \
+    }                                 \
+  } while (0)
+#else
+#define FA_TIMELINE_QK() ((void)0)
+#endif
+
 namespace fa {
 
 constexpr int kLoopPersistentMaxSeqs = 128;
@@ -54,12 +68,16 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   constexpr int SL = NR / NT;
   static_assert(NT > 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 2, "merge slices the output across wavefronts");
 
+  FA_TIMELINE_STAMP(0);
+  FA_TIMELINE_WHERE();
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int team = HPW == 1 ? 0 : wave / NT;   // which of the item's HPW adjacent kv heads
   const int tw = HPW == 1 ? wave : wave % NT;  // wavefront within the team
   const int G = gridDim.x;
   const int wg = blockIdx.x;
+  [[maybe_unused]] int timeline_chunks = 0;
+  [[maybe_unused]] bool timeline_first = true;
   const int col_max = p.max_blocks_per_seq - 1;
 
   // The items, (sequence, kv head) pairs with the longest sequences first, dealt in snake order;
@@ -88,6 +106,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
   int n = 0;
   Item cur;
   if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
+  FA_TIMELINE_STAMP(1);
   if constexpr (EXT) cur.c_lo = wa.first_visible_chunk(cur.ctx, 0);
   if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
@@ -217,6 +236,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
         {  // first chunk of the item, then the merge owed to the previous item
           const int cn = ci + NT;
           const auto s = wa.qk(R);
+          FA_TIMELINE_QK();
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.ctx, &ts);
@@ -233,6 +253,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
         while (ci + NT < cur.c_end) {  // steady state: the next chunk belongs to the same item
           const int cn = ci + NT;
           const auto s = wa.qk(R);
+          FA_TIMELINE_QK();
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.ctx, &ts);
@@ -245,6 +266,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       }
       // last chunk of this wavefront in `cur`: what goes out next belongs to `nxt`
       const auto s = wa.qk(R);
+      FA_TIMELINE_QK();
       if (next_armed) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
         next_sink = wa.load_sink(nxt.kvh, tw == 0);
@@ -261,6 +283,7 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
       wa.issue_v(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
       if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
+    if (!has_next) FA_TIMELINE_STAMP(3);
     if (owed) finish(n - 1, prev.seq, prev.kvh, prev_out_mul);
     publish(n);
 
@@ -277,6 +300,8 @@ paged_attn_loop_persistent_kernel(const PagedAttnParams p) {
     ++n;
   }
   finish(n, cur.seq, cur.kvh, EXT ? cur_ext.out_mul : 1.f);
+  FA_TIMELINE_STAMP(4);
+  FA_TIMELINE_PUT(5, timeline_chunks);
 }
 
 }  // namespace fa

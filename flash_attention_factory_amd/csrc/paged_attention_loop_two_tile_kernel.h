@@ -115,7 +115,7 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
   // Merge the NW published states of one tile of an item, normalise, store this wavefront's slice.
   // whole: the item is the row's only partial, which goes to the call's `out` as its result
   // (PagedAttnParams::final_out)
-  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool mark, bool whole, float out_mul) __attribute__((always_inline)) {
+  auto finish_tile = [&](W &w, int tile, int b, int seq, int kvh, int part0, bool whole, float out_mul) __attribute__((always_inline)) {
     const int w0 = team * NT;  // the team's wavefronts: w0 .. w0 + NT - 1
     float M = -INFINITY;
 #pragma unroll
@@ -153,7 +153,6 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
           for (int u = 0; u < NT; ++u) MT = fmaxf(MT, sm_mt[tile][b][w0 + u][i]);
           p.max_logits[slot] = MT * kLn2;  // natural-log units, as upstream stores them
           p.exp_sums[slot] = MT == -INFINITY ? 0.f : L * fast_exp2(M - MT);
-          if (mark) p.max_logits[slot + 1] = segment_mark(items.m);  // for the reduce kernel
         }
       } else {
         W::template store_q<SL>(reinterpret_cast<char *>(p.out) + ((row * p.num_heads + head) * D + d0) * 2, o, inv);
@@ -179,13 +178,20 @@ paged_attn_loop_two_tile_kernel(const PagedAttnParams p) {
     }
     if (!arrived && lane == 0) __hip_atomic_store(p.status, kStatusSpinLimit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    // a row of two or more partitions: its first segment leaves the segment length (segment_mark)
-    bool mark = false;
-    if constexpr (PART) mark = it.part0 == 0 && items.m > 1 && it.ctx > p.partition_size && p.max_num_partitions > 1;
     bool whole = false;
     if constexpr (PART) whole = p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx;
-    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, mark, whole, out_mul);
-    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, mark, whole, out_mul);
+    finish_tile(wa, 0, b, it.seq, it.kvh, it.part0, whole, out_mul);
+    finish_tile(wb, 1, b, it.seq, it.kvh, it.part0, whole, out_mul);
+    if constexpr (PART) {
+      // the slots that the piece covers beyond its first tell the reduce kernel that they hold no partial
+      if (tw == 0 && it.parts > 1) {
+        for (int q = 0; q < p.query_count; ++q) {
+          const int64_t row = (int64_t)it.seq * p.query_len + p.query_first + q;
+          mark_covered_slots(p.max_logits, (row * p.num_heads + (int64_t)it.kvh * p.group) * p.max_num_partitions + it.part0,
+                             p.group, p.max_num_partitions, it.parts, lane, items.m);
+        }
+      }
+    }
   };
   auto table_of = [&](int seq) __attribute__((always_inline)) { return p.block_tables + (int64_t)seq * p.max_blocks_per_seq; };
   // this wavefront's chunks of an item: c_lo + tw, + NW, ... below c_end

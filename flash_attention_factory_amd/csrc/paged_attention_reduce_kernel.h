@@ -5,8 +5,9 @@
 //   M = max_p m_p; w_p = l_p * exp(m_p - M)            (rescale_exp_sums :736-764)
 //   out = sum_p (w_p / sum_q w_q) * tmp_out[p, :]      (compute_out :771-864, collect_out :868-934)
 // Only the ceil(context_len / partition_size) live partitions are read (:679,716).
-// After the segment attention kernels a row of a single partial is left alone: the attention
-// kernel has stored it into `out` already.
+// After the segment attention kernels a partial may cover several partitions: it sits in the slot
+// of the first, the others hold a mark (paged_attention_segment_policy.h); and a row of a single
+// partial is left alone: the attention kernel has stored it into `out` already.
 //
 // One work-group of one or four wavefronts per (sequence, head).  The kernel is a chain
 // of dependent memory round trips, so it is built to have as few of them as possible:
@@ -38,9 +39,9 @@ struct ReduceParams {
   int32_t num_seqs;
   int32_t num_kv_heads;
   int32_t query_len;       // query tokens per sequence: rows of out / scratch are (sequence, query token) pairs
-  int32_t segment_groups;  // > 0: a segment attention kernel wrote the partials (one per segment of
-                           // m partitions, into the segment's first slot, and m into slot 1 of
-                           // max_logits: segment_mark); 0: one partial per partition
+  int32_t segment_groups;  // > 0: a segment attention kernel wrote the partials (one per piece of
+                           // several partitions, into the piece's first slot, marks into the
+                           // others: segment_mark); 0: one partial per partition
 };
 
 // Rows requested per wavefront and batch: 16 when every partition has a partial (dozens per
@@ -53,8 +54,10 @@ constexpr int reduce_rows_in_flight() { return SEGMENTS ? FA_REDUCE_SEGMENT_ROWS
 // pairs -- the launch is then short of parallelism and each pair's rows should be in
 // flight at once -- 1 when there are thousands and every wavefront slot of the GPU is
 // filled anyway (no LDS, no barrier, more groups resident).
-template <int D, typename QT, int kReduceWaves, bool SEGMENTS = false>
-__global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
+// Every live slot holds a partial (the grid form of the attention kernels).
+template <int D, typename QT, int kReduceWaves>
+__device__ __forceinline__ void reduce_every_partition(const ReduceParams &p) {
+  constexpr bool SEGMENTS = false;
   constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
   constexpr int R = reduce_rows_in_flight<SEGMENTS>();
   const int lane = threadIdx.x & 63;
@@ -64,25 +67,11 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
   const int seq = blockIdx.x / p.num_heads;
   const int head = blockIdx.x - seq * p.num_heads;
   const int64_t base = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions;
-  // Partials lie `stride` slots apart: 1, or the segment length the attention kernel chose and left
-  // in slot 1 of the row (segment_mark).  Requested together with the length, whether or not the
-  // row turns out to have a second partition, so that one wait covers both.
-  float slot1 = 0.f;
-  if constexpr (SEGMENTS) {
-    if (p.max_num_partitions > 1) slot1 = p.max_logits[base + 1];
-  }
   const int ctx = min(p.context_lens[p.query_len > 1 ? seq / p.query_len : seq], p.max_context);
   if (ctx <= 0) return;
   int np = (ctx + p.partition_size - 1) / p.partition_size;
   np = min(np, p.max_num_partitions);
-  int stride = 1;
-  if constexpr (SEGMENTS) {
-    if (np > 1) stride = __builtin_amdgcn_readfirstlane(segment_length_of(slot1));
-    np = (np + stride - 1) / stride;  // from here on: the number of partials
-    // one partial: the segment kernel has stored it into `out` as the row's result
-    // (PagedAttnParams::final_out), and its tmp_out row holds nothing
-    if (np == 1) return;
-  }
+  constexpr int stride = 1;
   const float *ml = p.max_logits + base;
   const float *es = p.exp_sums + base;
   const float *tmp = p.tmp_out + base * D + lane * EPL;
@@ -160,6 +149,132 @@ __global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(co
     const uint32_t w = pack2<QT>(o[0], 0.f);
     *reinterpret_cast<uint16_t *>(dst) = (uint16_t)(w & 0xffffu);
   }
+}
+
+
+// Partials wherever a slot does not hold the mark of a covered slot (the segment attention kernels).
+template <int D, typename QT, int kReduceWaves>
+__device__ __forceinline__ void reduce_marked_partials(const ReduceParams &p) {
+  constexpr bool SEGMENTS = true;
+  constexpr int EPL = D / 64;  // output elements per lane (2 or 1)
+  constexpr int R = reduce_rows_in_flight<SEGMENTS>();
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // one work-group per (row, head), heads fastest; a row of out and of the scratch arrays is a
+  // sequence, or a (sequence, query token) pair
+  const int seq = blockIdx.x / p.num_heads;
+  const int head = blockIdx.x - seq * p.num_heads;
+  const int64_t base = ((int64_t)seq * p.num_heads + head) * p.max_num_partitions;
+  const float *ml = p.max_logits + base;
+  const float *es = p.exp_sums + base;
+  const float *tmp = p.tmp_out + base * D + lane * EPL;
+  // The scalars of the row's first 64 slots are requested together with the length, whether or not
+  // the row turns out to have that many partitions, so that one wait covers both (slots past the
+  // live ones are read and dropped: they lie inside the row).
+  const int first_slots = min(p.max_num_partitions, 64);
+  const float ml_first = lane < first_slots ? ml[lane] : -INFINITY;
+  const float es_first = lane < first_slots ? es[lane] : 0.f;
+  const int ctx = min(p.context_lens[p.query_len > 1 ? seq / p.query_len : seq], p.max_context);
+  if (ctx <= 0) return;
+  int np = (ctx + p.partition_size - 1) / p.partition_size;
+  np = min(np, p.max_num_partitions);
+  // After a segment attention kernel a slot holds a partial unless it holds the mark of a slot that a
+  // longer piece covers (segment_mark); after the grid form every live slot holds a partial.
+  auto holds_partial = [&](int q, float m_q) { return q < np && !(SEGMENTS && is_segment_mark(m_q)); };
+  if constexpr (SEGMENTS) {
+    // one partial: the segment kernel has stored it into `out` as the row's result
+    // (PagedAttnParams::final_out), and its tmp_out row holds nothing
+    if (np == 1) return;
+  }
+
+  // Partitions are handled in groups of 64 (lane q of the wavefront holds the weight of
+  // partition 64g + q).  First the maximum over all partials, and how many there are.
+  float M = holds_partial(lane, ml_first) ? ml_first : -INFINITY;
+  int partials = __builtin_popcountll(__ballot(holds_partial(lane, ml_first)));
+  for (int g0 = 64; g0 < np; g0 += 64) {
+    const float m_q = g0 + lane < np ? ml[g0 + lane] : -INFINITY;
+    const bool there = holds_partial(g0 + lane, m_q);
+    if (there) M = fmaxf(M, m_q);
+    partials += __builtin_popcountll(__ballot(there));
+  }
+  if constexpr (SEGMENTS) {
+    if (partials <= 1) return;  // a row that one piece covers: stored into `out` by the attention kernel
+  }
+  M = wave_max(M);
+  // a row none of whose partitions saw a key (a query token placed before key 0): every
+  // max is -inf and every sum 0; keep exp(m - M) finite so that the row comes out as zeros
+  if (M == -INFINITY) M = 0.f;
+
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+  float W = 0.f;
+  int nth = 0;  // partials met so far: wavefront w takes those with nth % kReduceWaves == w
+  for (int g0 = 0; g0 < np; g0 += 64) {
+    const int ql = g0 + lane;
+    const float m_q = g0 == 0 ? ml_first : (ql < np ? ml[ql] : -INFINITY);
+    const bool there = holds_partial(ql, m_q);
+    const float e_q = g0 == 0 ? es_first : (there ? es[ql] : 0.f);
+    const float w_lane = there ? e_q * __expf(m_q - M) : 0.f;
+    W += w_lane;
+    unsigned long long todo = __ballot(there);
+    while (todo) {  // wave-uniform: R rows of tmp_out per wavefront in flight at a time
+      int slot[R];
+      float v[R][EPL];
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        slot[u] = -1;
+        while (todo && slot[u] < 0) {
+          const int q = __builtin_ctzll(todo);
+          todo &= todo - 1;
+          if ((nth++ % kReduceWaves) == wave) slot[u] = q;
+        }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) v[u][e] = slot[u] >= 0 ? tmp[(int64_t)(g0 + slot[u]) * D + e] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const float w = slot[u] >= 0 ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_lane), __builtin_amdgcn_readfirstlane(slot[u]))) : 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[e] += w * v[u][e];
+      }
+    }
+  }
+  W = wave_sum(W);
+
+  const float inv = W > 0.f ? 1.0f / W : 0.f;
+  float o[EPL];
+  if constexpr (kReduceWaves == 1) {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) o[e] = acc[e] * inv;
+  } else {
+    __shared__ float part[kReduceWaves][D];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) part[wave][lane * EPL + e] = acc[e];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      float a = 0.f;
+#pragma unroll
+      for (int w = 0; w < kReduceWaves; ++w) a += part[w][lane * EPL + e];
+      o[e] = a * inv;
+    }
+  }
+  char *dst = reinterpret_cast<char *>(p.out) +
+              (((int64_t)seq * p.num_heads + head) * D + lane * EPL) * 2;
+  if constexpr (EPL == 2) {
+    *reinterpret_cast<uint32_t *>(dst) = pack2<QT>(o[0], o[1]);
+  } else {
+    const uint32_t w = pack2<QT>(o[0], 0.f);
+    *reinterpret_cast<uint16_t *>(dst) = (uint16_t)(w & 0xffffu);
+  }
+}
+
+template <int D, typename QT, int kReduceWaves, bool SEGMENTS = false>
+__global__ void __launch_bounds__(kReduceWaves * 64) paged_attn_reduce_kernel(const ReduceParams p) {
+  if constexpr (SEGMENTS) reduce_marked_partials<D, QT, kReduceWaves>(p);
+  else reduce_every_partition<D, QT, kReduceWaves>(p);
 }
 
 }  // namespace fa

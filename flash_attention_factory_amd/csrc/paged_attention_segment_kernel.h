@@ -9,8 +9,8 @@
 // of m consecutive partitions of one (sequence, kv head): its wavefronts interleave the
 // segment's chunks, merge their states in LDS (no barrier: the deferred merge of the
 // persistent loop kernel) and write ONE partial into the slot of the segment's first
-// partition.  Of the other m - 1 slots only slot 1 of max_logits is written, with m itself
-// (segment_mark): the reduce kernel reads it there and visits slots 0, m, 2m, ...
+// partition.  The other m - 1 slots of max_logits get a mark (segment_mark) by which the reduce
+// kernel tells them from slots that hold partials.
 // A sequence that fits one segment has one partial, which is its result: that one is rounded to
 // the query type and stored into the call's `out` (PagedAttnParams::final_out), its scalars into
 // exp_sums and max_logits as ever, and the reduce kernel leaves the row alone -- in a batch of
@@ -19,9 +19,11 @@
 // m is chosen on the device from the batch itself -- every wavefront evaluates
 // partitions_per_segment() on the same context lengths -- so that a segment is about what a
 // compute unit, or a work-group of it, should stream: a batch of few long sequences gets one
-// segment per unit or per work-group, in a batch with a thousand (sequence, kv head) pairs most
-// sequences stay whole.
-// Segments are dealt to the work-groups longest first in snake order (see below).
+// segment per unit or per work-group.  Segments are dealt to the work-groups longest first in
+// snake order (see below).  On request (options->segment_partitions = -1) a batch is cut differently,
+// into even shares: the rows laid end to end, one contiguous share per work-group, so that a
+// work-group's pieces are the end of one row, whole rows and the beginning of another
+// (paged_attention_segment_policy.h).
 // Built for up to 256 sequences; larger batches use the grid form.
 //
 // EXT: the extended instance (score modifiers, several query tokens per sequence, per-head or
@@ -56,11 +58,15 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   static_assert(NT > 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 4 && SL % 4 == 0,
                 "each wavefront stores whole 16-byte pieces");
 
+  FA_TIMELINE_STAMP(0);
+  FA_TIMELINE_WHERE();
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int team = HPW == 1 ? 0 : wave / NT;   // which of the item's HPW adjacent kv heads
   const int tw = HPW == 1 ? wave : wave % NT;  // wavefront within the team
   const int G = gridDim.x;
+  [[maybe_unused]] int timeline_chunks = 0;
+  [[maybe_unused]] bool timeline_first = true;
   const int col_max = p.max_blocks_per_seq - 1;
 
   // The segment list (SegmentItems): all full segments, then the sequences' last, shorter segments
@@ -85,6 +91,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
 
   Item cur;
   if (!item_at(0, cur)) return;  // the same for every wavefront of the work-group
+  FA_TIMELINE_STAMP(1);
   if (threadIdx.x < 2) sm_arrived[threadIdx.x] = 0;
   __syncthreads();  // the only barrier: wavefronts meet through the counters from here on
 
@@ -169,10 +176,15 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       if ((wa.paired() ? (r & 1) == 0 : r == 0) && tw == 0) {  // one lane per column, see merge_and_store
         p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
         p.exp_sums[slot] = L;
-        // the first segment of a row of two or more partitions tells the reduce kernel how long
-        // segments are (segment_mark)
-        if (it.part0 == 0 && items.m > 1 && it.ctx > p.partition_size && p.max_num_partitions > 1)
-          p.max_logits[slot + 1] = segment_mark(items.m);
+      }
+    }
+    // the slots that the piece covers beyond its first tell the reduce kernel that they hold no partial
+    if (tw == 0 && it.parts > 1) {
+      const int rows = EXT ? p.query_count : 1;  // query tokens of the launch
+      for (int q = 0; q < rows; ++q) {
+        const int64_t row = EXT ? (int64_t)it.seq * p.query_len + p.query_first + q : it.seq;
+        mark_covered_slots(p.max_logits, (row * p.num_heads + (int64_t)it.kvh * p.group) * p.max_num_partitions + it.part0,
+                           p.group, p.max_num_partitions, it.parts, lane, items.m);
       }
     }
   };
@@ -224,6 +236,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
         {  // first chunk of the item, then the merge owed to the previous item
           const int cn = ci + NT;
           const auto s = wa.qk(R);
+          FA_TIMELINE_QK();
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
@@ -240,6 +253,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
         while (ci + NT < cur.c_end) {  // steady state: the next chunk belongs to the same item
           const int cn = ci + NT;
           const auto s = wa.qk(R);
+          FA_TIMELINE_QK();
           wa.issue_k(R, cur.kvh, cn, nids);
           if constexpr (EXT) nts = wa.fetch_scales(nids, cur.kvh, cur_ext);
           const auto pb = wa.template soft<false, EXT>(R, s, ci, cur.tok_end, &ts);
@@ -252,6 +266,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       }
       // last chunk of this wavefront in `cur`: what goes out next belongs to `nxt`
       const auto s = wa.qk(R);
+      FA_TIMELINE_QK();
       if (next_armed) {
         wa.load_q(nxt.seq, nxt.kvh);  // Q registers are free once the last scores are out
         next_sink = wa.load_sink(nxt.kvh, tw == 0 && nxt.part0 == 0);
@@ -268,6 +283,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       wa.issue_v(R, nxt.kvh, nxt.c_lo + tw, nxt_ids);
       if constexpr (EXT) nxt_ts = wa.fetch_scales(nxt_ids, nxt.kvh, nxt_ext);
     }
+    if (!has_next) FA_TIMELINE_STAMP(3);
     if (owed) finish(n - 1, prev, prev_out_mul);
     publish(n);
 
@@ -284,6 +300,8 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     ++n;
   }
   finish(n, cur, EXT ? cur_ext.out_mul : 1.f);
+  FA_TIMELINE_STAMP(4);
+  FA_TIMELINE_PUT(5, timeline_chunks);
 }
 
 }  // namespace fa

@@ -1,9 +1,15 @@
 // How the segment form of the split path cuts sequences.  The attention kernels
 // (paged_attention_segment_kernel.h, the split form of paged_attention_loop_two_tile_kernel.h)
-// choose the segment length from the batch, every wavefront for itself, and write one partial per
-// segment into the slot of the segment's first partition; the reduce kernel
-// (paged_attention_reduce_kernel.h) finds the length in the scratch arrays: a length other than 1
-// leaves slot 1 of every row free, and there the attention kernel leaves a mark (segment_mark).
+// choose the cuts from the batch, every wavefront for itself, and write one partial per piece into
+// the slot of the piece's first partition.  Two ways of cutting:
+//   segments     every row is cut into segments of m partitions (partitions_per_segment), the
+//                segments are dealt to the work-groups longest first;
+//   even shares  (on request) the rows, laid end to end, are cut into one contiguous share per
+//                work-group, equal in keys (plus a cost per piece) to within half a partition: a
+//                work-group's pieces are the end of one row, whole rows, and the beginning of another.
+// The reduce kernel (paged_attention_reduce_kernel.h) finds the pieces in the scratch arrays
+// themselves: every slot of max_logits that a piece covers beyond its first holds a mark
+// (segment_mark), a NaN no maximum can be.
 #pragma once
 
 #include "paged_attention_utils.h"
@@ -41,6 +47,19 @@ __device__ __forceinline__ int wave_total(int v) {
   return __builtin_amdgcn_readfirstlane(__reduce_add_sync(~0ull, v));
 }
 
+// Inclusive prefix sum over the 64 lanes, in data-parallel-primitive moves: shifts by 1, 2, 4 and 8
+// within each row of 16 lanes (lanes shifted in from outside a row read 0), then the total of row 0
+// onto row 1 and of row 2 onto row 3, then that of rows 0-1 onto rows 2-3.
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, true);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, true);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, true);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, true);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Segment length as a share (in 1/1024) of a compute unit's mean load, against the sequences
 // per compute unit (in 1/1024).  Every sequence ends in a segment shorter than the others, so
 // with many sequences per compute unit the short ones alone fill the GPU and only sequences well
@@ -59,19 +78,46 @@ __device__ __forceinline__ int segment_share_of_load(int seqs_per_cu_1024) {
   return 360;
 }
 
-// The mark in max_logits[row][1]: a NaN no maximum can be (maxima are finite or -inf, and a NaN
-// that arithmetic makes has none of the low mantissa bits set), the segment length in its low
-// byte.  Rows of one partition need none; with a segment length of 1 slot 1 holds a partial.
+// The mark in the slots of max_logits that a piece covers beyond its first: a NaN no maximum can be
+// (maxima are finite or -inf, and a NaN that arithmetic makes has none of the low mantissa bits
+// set); in its low byte the segment length m, or 0 under even shares (for whoever inspects the
+// arrays: the reduce kernel only asks whether a slot holds a mark).
 constexpr uint32_t kSegmentMarkBits = 0x7FD3A600u, kSegmentMarkMask = 0xFFFFFF00u;
 static_assert(kSegmentMaxPartitions < 256, "the segment length is kept in one byte of the mark");
 __device__ __forceinline__ float segment_mark(int m) { return __uint_as_float(kSegmentMarkBits | (uint32_t)m); }
-// segment length a row's slot 1 tells: 1 unless it holds the mark
-__device__ __forceinline__ int segment_length_of(float slot1) {
-  const uint32_t bits = __float_as_uint(slot1);
-  if ((bits & kSegmentMarkMask) != kSegmentMarkBits) return 1;
-  return max(1, min((int)(bits & 0xFFu), kSegmentMaxPartitions));
+__device__ __forceinline__ bool is_segment_mark(float slot) {
+  return (__float_as_uint(slot) & kSegmentMarkMask) == kSegmentMarkBits;
 }
 
+// Marks the slots that a piece of `parts` partitions covers beyond its first, in the max_logits rows
+// of `heads` consecutive heads; first_slot: the piece's own slot in the first of these rows;
+// pitch: slots per row.  One wavefront, all lanes.
+__device__ __forceinline__ void mark_covered_slots(float *max_logits, int64_t first_slot, int heads, int pitch,
+                                                   int parts, int lane, int low_byte) {
+  const float mark = segment_mark(low_byte);
+  for (int h = 0; h < heads; ++h)
+    for (int q = 1 + lane; q < parts; q += 64) max_logits[first_slot + (int64_t)h * pitch + q] = mark;
+}
+
+// Even shares are cut on request only (options->segment_partitions = -1).  They give every work-group
+// the same number of keys to within half a partition, where dealing sorted segments leaves the most
+// loaded compute unit of a serving mix 7-10 % above the mean -- and yet, measured on 130 batches of 1 to
+// 256 sequences (both cache types, log-normal, long and short rows), segments are as fast or faster in
+// nine of ten, by 1-7 % on the large mixes: what a compute unit streams is not a matter of keys alone.
+// The older of a unit's two work-groups is served first and wants the larger share, rows of a few hundred
+// keys cost more per key than long ones, and the fitted segment rule has both in it.
+// The unit the shares are counted in: keys of one row, 32 at a time (what a wavefront takes at a time);
+// and what a piece costs beyond its keys, in the same unit.
+constexpr int kShareTokensLog2 = 5, kShareTokens = 1 << kShareTokensLog2;
+#ifndef FA_SHARE_PIECE_COST
+#define FA_SHARE_PIECE_COST 4
+#endif
+constexpr int kSharePieceCost = FA_SHARE_PIECE_COST;
+// With two work-groups per compute unit: what the older one of a unit takes of the unit's work, in 1/1000.
+#ifndef FA_SHARE_OLDER_PERMILLE
+#define FA_SHARE_OLDER_PERMILLE 540
+#endif
+constexpr int kShareOlderPermille = FA_SHARE_OLDER_PERMILLE;
 // Whole segments and segments in all (per kv head) that a segment length of m partitions
 // leaves: lane holds sequences lane, lane + 64, ... of which ctxv / parts are the lengths and
 // live partitions.

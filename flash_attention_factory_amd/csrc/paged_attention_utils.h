@@ -26,6 +26,33 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 struct F16 {};   // query / output element tags
 struct BF16 {};
 
+// ---- in-kernel timeline (debug builds with -DFA_TIMELINE only) -------------------------------------
+// Wall-clock stamps (the 100 MHz counter of s_memrealtime) that wavefronts of the persistent kernels
+// leave in a device array, eight 64-bit slots per wavefront; fa_debug_timeline() copies it to the host.
+// Slots: 0 kernel entry, 1 lengths in and items ranked, 2 first K tile in registers, 3 last chunk
+// done, 4 last merge stored, 5 chunks this wavefront ran, 6 HW_ID register, 7 XCC_ID register.
+// Compiled out of the product library.
+#ifdef FA_TIMELINE
+constexpr int kTimelineWaves = 8192, kTimelineSlots = 8;
+static __device__ unsigned long long timeline_words[kTimelineWaves * kTimelineSlots];
+__device__ __forceinline__ void timeline_put(int slot, unsigned long long value) {
+  const int wave = (int)blockIdx.x * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6);
+  if ((threadIdx.x & 63) == 0 && wave < kTimelineWaves) timeline_words[wave * kTimelineSlots + slot] = value;
+}
+__device__ __forceinline__ void timeline_stamp(int slot) { timeline_put(slot, wall_clock64()); }
+__device__ __forceinline__ void timeline_where() {
+  timeline_put(6, __builtin_amdgcn_s_getreg((31 << 11) | 4));   // HW_ID
+  timeline_put(7, __builtin_amdgcn_s_getreg((31 << 11) | 20));  // XCC_ID
+}
+#define FA_TIMELINE_STAMP(slot) ::fa::timeline_stamp(slot)
+#define FA_TIMELINE_PUT(slot, value) ::fa::timeline_put(slot, (unsigned long long)(value))
+#define FA_TIMELINE_WHERE() ::fa::timeline_where()
+#else
+#define FA_TIMELINE_STAMP(slot) ((void)0)
+#define FA_TIMELINE_PUT(slot, value) ((void)0)
+#define FA_TIMELINE_WHERE() ((void)0)
+#endif
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

@@ -84,7 +84,7 @@ struct PagedAttnParams {
   // contiguous)
   int32_t compute_units;
   int32_t kv_rows_apart;
-  int32_t segment_force;  // > 0: partitions per segment as the caller fixed them (options->segment_partitions)
+  int32_t segment_force;  // options->segment_partitions: > 0 partitions per segment as the caller fixed them, -1 even shares
   // Split path, segment form: the call's `out`.  A row whose context fits one segment has one
   // partial, which is its result: the attention kernel rounds it to the query type and stores it
   // here, not into tmp_out (exp_sums and max_logits still get the partial's scalars), and the reduce

@@ -188,9 +188,11 @@ typedef struct fa_paged_attention_options {
                                  void, see fa_paged_attention_kernel_status).  0 = the library's bound,
                                  which no correct run reaches; negative = do not wait at all, which makes
                                  the give-up path run for a test while every kernel still ends normally */
-  int32_t segment_partitions; /* reduce entries, FA_SCHEDULE_AUTO: partitions that one partial covers where
-                                 the library would choose that number itself (see fa_paged_attention_reduce);
-                                 0 = the library chooses, n >= 1 = n (at most 64).  A tuning and test knob:
+  int32_t segment_partitions; /* reduce entries, FA_SCHEDULE_AUTO: how rows are cut into partials where the
+                                 library would choose that itself (see fa_paged_attention_reduce): 0 = the
+                                 library chooses; n >= 1 = every n partitions (at most 64); -1 = even shares,
+                                 one contiguous run of partitions per work-group; -2 = segments of the length
+                                 the library's rule gives, never even shares.  A tuning and test knob:
                                  `out` does not depend on it beyond the order of fp32 sums */
 } fa_paged_attention_options;
 #define FA_PAGED_ATTENTION_OPTIONS_INIT {(uint32_t)sizeof(fa_paged_attention_options)}
@@ -207,11 +209,13 @@ int32_t fa_paged_attention_loop(void *out, const void *query, const void *key_ca
  * scratch the two kernels hand partial softmax states through; every slot either holds what
  * upstream stores there for its partition -- or nothing: for batches with many
  * (sequence, kv head) pairs one partial covers several consecutive partitions and sits in
- * the slot of the first; of the slots in between, slot 1 of max_logits then tells the reduce
- * kernel how many partitions a partial covers (a NaN with that number in its low byte), the
- * others stay untouched; and a row whose whole context lies in one partial gets that partial
- * straight into `out`, as its result -- its scalars are in exp_sums and max_logits, its tmp_out
- * row stays untouched.  Only `out` is a result. */
+ * the slot of the first; the slots of max_logits in between hold a mark by which the reduce
+ * kernel tells them from partials (a NaN no maximum can be), those of exp_sums and tmp_out stay
+ * untouched; a row whose whole context lies in one partial gets that partial straight into `out`,
+ * as its result -- its scalars are in exp_sums and max_logits, its tmp_out row stays untouched; and
+ * where the rows are provably too short for splitting to pay the call runs the single-pass kernel
+ * and leaves all three arrays alone (fa_paged_attention_reduce_plan).  Only `out` is a result;
+ * FA_SCHEDULE_GRID is the schedule under which the arrays hold upstream's per-partition contents. */
 int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_cache,
                                   const void *value_cache, const int32_t *block_tables,
                                   const int32_t *context_lens, float scale,

@@ -109,6 +109,57 @@ def partitions_per_segment(lens, *, partition_size: int, max_num_partitions: int
     return before if before > 0 else m
 
 
+SHARE_TOKENS = 32
+SHARE_PIECE_COST = 4
+
+
+def even_shares_pieces(lens, *, partition_size: int, max_num_partitions: int, max_ctx: int, num_kv_heads: int,
+                       groups: int, cus: int):
+    """The pieces even shares cut the batch into: {(sequence, kv-head item): [(first partition, partitions,
+    work-group), ...]} -- what options->segment_partitions = -1 asks for.  A row costs its keys in steps
+    of 32 plus 4 steps; the rows' costs lie end to end, sequences in order and kv heads within a sequence;
+    the work-groups take equal stretches of that tape in turn (to within a step; with two work-groups on
+    every compute unit the older half of them takes 54 % of it), and what a work-group holds of a row
+    runs between the partition boundaries nearest to its stretch's ends
+    (csrc/paged_attention_items.h: build_even_shares, next_of_share)."""
+    ctx, parts = live_partitions(lens, partition_size, max_num_partitions, max_ctx)
+    ctx = [min(c, p * partition_size) for c, p in zip(ctx, parts)]
+    cost = [(c + SHARE_TOKENS - 1) // SHARE_TOKENS + SHARE_PIECE_COST if c > 0 else 0 for c in ctx]
+    n = sum(cost) * num_kv_heads
+    # two work-groups per compute unit (g and g + cus): the older half takes 540 / 1000 of the tape
+    halves = [(0, n, groups)]
+    if groups == 2 * cus:
+        older = int(F(n) * (F(540) * F(0.001)))
+        halves = [(0, older, cus), (older, n - older, cus)]
+    bounds = []
+    for begin, length, count in halves:
+        each, extra = divmod(length, count)
+        bounds += [begin + g * each + min(g, extra) for g in range(count)]
+    bounds.append(n)
+    steps = partition_size // SHARE_TOKENS
+
+    def nearest_cut(x, parts_of_row):
+        return min(parts_of_row, (x + steps // 2) // steps)
+
+    pieces = {}
+    row_begin = 0
+    for s, (c, p) in enumerate(zip(cost, parts)):
+        for k in range(num_kv_heads if c else 0):
+            row_end = row_begin + c
+            row = []
+            for g in range(groups):
+                lo, hi = bounds[g], bounds[g + 1]
+                if hi <= row_begin or lo >= row_end or lo == hi:
+                    continue
+                first = 0 if lo <= row_begin else nearest_cut(lo - row_begin, p)
+                last = p if hi >= row_end else nearest_cut(hi - row_begin, p)
+                if last > first:
+                    row.append((first, last - first, g))
+            pieces[(s, k)] = row
+            row_begin = row_end
+    return pieces
+
+
 def segments_of(lens, m: int, *, partition_size: int, max_num_partitions: int, max_ctx: int):
     """Token lengths of the segments a length of m partitions cuts the batch into (per kv head)."""
     ctx, parts = live_partitions(lens, partition_size, max_num_partitions, max_ctx)

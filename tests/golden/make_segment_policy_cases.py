@@ -63,8 +63,11 @@ def batches(seed: int, per_shape: int = 9):
     return out
 
 
-def device_choice(case, dev):
-    """(m the attention kernel chose or None if no row has two partitions, plan) for one batch."""
+def device_choice(case, dev, segment_partitions=0):
+    """(how the attention kernel cut the batch, plan, the slots of every (sequence, kv-head item) row that
+    hold partials) for one batch.  The cut: m, the partitions per segment; 0 for even shares
+    (segment_partitions = -1); None if the call did not run in the segment form or no slot holds a mark
+    (no piece covers two partitions)."""
     from flash_attention_factory_amd import _cabi, lib
     d, hk, group, block, psize = (case[k] for k in ("head_size", "num_kv_heads", "group", "block_size", "partition_size"))
     lens = torch.tensor(case["lens"], dtype=torch.int32)
@@ -87,7 +90,7 @@ def device_choice(case, dev):
     head = [ml, es, tmp, out, None, query, view(key), view(value), tables, lens.to(dev), group, d ** -0.5]
     if case["fp8"]:
         head.append(1.0)
-    mod.run(*head, block, 0, None, None, 0.0, partition_size=psize, timed=False)
+    mod.run(*head, block, 0, None, None, 0.0, partition_size=psize, timed=False, segment_partitions=segment_partitions)
     torch.cuda.synchronize()
     # the plan of the same call
     sh = _cabi.Shape()
@@ -98,35 +101,65 @@ def device_choice(case, dev):
     sh.q_dtype, sh.num_pool_blocks = _cabi.FA_DTYPE_F16, nb
     plan = _cabi.SplitPlan()
     _cabi.check(_cabi.load().fa_paged_attention_reduce_plan(ctypes.byref(sh), None, 0, int(case["fp8"]), 0, ctypes.byref(plan)))
-    longest = int(lens.argmax())
-    m = None
-    if plan.form == _cabi.FA_SPLIT_FORM_SEGMENT and int(lens.max()) > psize:
-        bits = int(ml[longest, 0, 1].view(torch.int32).item()) & 0xFFFFFFFF
-        m = (bits & 0xFF) if (bits & MARK_MASK) == MARK_BITS else 1
+    m, slots = None, {}
+    if plan.form == _cabi.FA_SPLIT_FORM_SEGMENT:
+        bits = ml.view(torch.int32).cpu()
+        marks = bits[(bits & MARK_MASK) == MARK_BITS]
+        if marks.numel():
+            low = set((marks & 0xFF).tolist())
+            assert len(low) == 1, low  # every mark of a launch carries the same byte
+            m = low.pop()
+        first_head = plan.kv_heads_per_item * group  # query heads per kv-head item
+        written = ~torch.isnan(ml.cpu())
+        for s in range(S):
+            for k in range(hk // plan.kv_heads_per_item):
+                if case["lens"][s] > 0:
+                    slots[(s, k)] = torch.nonzero(written[s, k * first_head]).flatten().tolist()
     return m, dict(form=plan.form, compute_units=plan.compute_units, work_groups=plan.work_groups,
-                   kv_heads_per_item=plan.kv_heads_per_item)
+                   kv_heads_per_item=plan.kv_heads_per_item), slots
 
 
-def replay(case, plan):
-    """The same choice by the host restatement of the rule."""
+def _policy():
     sys.path.insert(0, os.path.dirname(HERE))
-    import _segment_policy as P
+    import _segment_policy
+    return _segment_policy
+
+
+def _geometry(case, plan):
     d, hk, block, psize = (case[k] for k in ("head_size", "num_kv_heads", "block_size", "partition_size"))
     lens = case["lens"]
     mb = max(1, math.ceil(max(lens) / block))
     npart = max(1, math.ceil(max(lens) / psize))
     per_item = plan["kv_heads_per_item"]
-    row_bytes = d * (1 if case["fp8"] else 2) * per_item
-    return P.partitions_per_segment(lens, partition_size=psize, max_num_partitions=npart, max_ctx=mb * block,
-                                    num_kv_heads=hk // per_item, groups=plan["work_groups"], cus=plan["compute_units"],
-                                    rows_apart=case["token_major"], partition_bytes=2 * psize * row_bytes)
+    return dict(partition_size=psize, max_num_partitions=npart, max_ctx=mb * block, num_kv_heads=hk // per_item,
+                groups=plan["work_groups"])
+
+
+def replay(case, plan):
+    """The same choice by the host restatement of the rule: partitions per segment."""
+    P = _policy()
+    geo = _geometry(case, plan)
+    row_bytes = case["head_size"] * (1 if case["fp8"] else 2) * plan["kv_heads_per_item"]
+    return P.partitions_per_segment(case["lens"], cus=plan["compute_units"], rows_apart=case["token_major"],
+                                    partition_bytes=2 * case["partition_size"] * row_bytes, **geo)
+
+
+def replay_slots(case, plan, m):
+    """The slots that hold partials, per (sequence, kv-head item) row, for a cut of m (0: even shares)."""
+    P = _policy()
+    geo = _geometry(case, plan)
+    if m == 0:
+        pieces = P.even_shares_pieces(case["lens"], cus=plan["compute_units"], **geo)
+        return {row: [first for first, _, _ in cut] for row, cut in pieces.items()}
+    _, parts = P.live_partitions(case["lens"], geo["partition_size"], geo["max_num_partitions"], geo["max_ctx"])
+    return {(s, k): list(range(0, p, m)) for s, p in enumerate(parts) if p > 0 for k in range(geo["num_kv_heads"])}
 
 
 def main():
     dev = torch.device("cuda:0")
     cases = []
     for case in batches(seed=0):
-        m, plan = device_choice(case, dev)
+        m, plan, _ = device_choice(case, dev)
         if m is None:
             continue
         cases.append(dict(case, plan=plan, partitions_per_segment=m))

@@ -330,38 +330,79 @@ def _segment_batches(name):
     return w, "fp8_reduce"
 
 
-@pytest.mark.parametrize("name", ["one_segment_per_unit", "three_groups_per_unit", "longest_segment", "many_sequences"])
+def _split_plan(wd, kernel):
+    """fa_paged_attention_reduce_plan of the call runner.run_workload makes for this workload."""
+    import ctypes
+    from flash_attention_factory_amd import _cabi, runner
+    kc = runner.logical_cache_view(wd, wd.key_cache)
+    sh = _cabi.Shape()
+    sh.num_seqs, sh.num_heads, sh.head_size = wd.query.shape
+    sh.num_kv_heads, sh.block_size = wd.num_kv_heads, wd.block_size
+    sh.max_blocks_per_seq, sh.max_num_partitions, sh.partition_size = wd.block_tables.shape[1], wd.max_num_partitions, wd.partition_size
+    sh.kv_block_stride, sh.kv_token_stride, sh.kv_head_stride = kc.stride(0), kc.stride(1), kc.stride(2)
+    sh.q_dtype = _cabi.FA_DTYPE_BF16 if wd.query.dtype == torch.bfloat16 else _cabi.FA_DTYPE_F16
+    sh.num_pool_blocks = kc.size(0)
+    plan = _cabi.SplitPlan()
+    _cabi.check(_cabi.load().fa_paged_attention_reduce_plan(ctypes.byref(sh), None, 0, int(kernel.startswith("fp8")), 0,
+                                                            ctypes.byref(plan)))
+    return plan
+
+
+@pytest.mark.parametrize("name", ["one_segment_per_unit", "three_groups_per_unit", "longest_segment", "many_sequences",
+                                  "even_shares"])
 def test_segment_length_regimes(oracle, name):
-    """One batch for each way the split path arrives at its segment length (one segment per compute
-    unit; half a work-group's load where three share a unit; the cap of 64 partitions; a share of a
-    unit's load with many sequences): the output matches the oracle, every row of two or more
-    partitions carries the same mark, and exactly the slots 0, m, 2m, ... of its live partitions
-    hold partials."""
+    """One batch for each way the split path arrives at its cuts (one segment per compute unit; half a
+    work-group's load where three share a unit; the cap of 64 partitions; a share of a unit's load with
+    many sequences; even shares on request): the output matches the oracle, every mark of the launch
+    tells the same cut, and exactly the slots that cut names hold partials -- 0, m, 2m, ... of a row's
+    live partitions for segments, the starts of the work-groups' shares and of the rows for even shares."""
+    import _segment_policy as SP
+    forced = 0
+    if name == "even_shares":
+        name, forced = "many_sequences", -1
     w, kernel = _segment_batches(name)
     from flash_attention_factory_amd import runner
     wd = w.to(_dev())
     bufs = runner.alloc_buffers(wd)
     for t in (bufs.exp_sums, bufs.max_logits, bufs.tmp_out):
         t.fill_(float("nan"))
-    runner.run_workload(wd, kernel, bufs)
+    runner.run_workload(wd, kernel, bufs, segment_partitions=forced)
     torch.cuda.synchronize()
     _check(bufs.out, w, oracle, f"segment lengths, {name}")
     es = bufs.exp_sums.cpu()
     ml = bufs.max_logits.cpu()
     P = w.partition_size
     lens = [int(n) for n in w.context_lens.tolist()]
-    marks = {_segment_mark(ml[s, 0, 1]) for s in range(len(lens)) if lens[s] > P}
-    assert len(marks) == 1, marks
-    m = marks.pop() or 1
-    print(f"{name}: {m} partitions per segment", flush=True)
-    if name == "longest_segment":
+    bits = ml.view(torch.int32)
+    marks = set((bits[(bits & 0xFFFFFF00) == 0x7FD3A600] & 0xFF).tolist())
+    assert len(marks) <= 1, marks
+    m = marks.pop() if marks else 1
+    print(f"{name}: " + (f"{m} partitions per segment" if m else "even shares"), flush=True)
+    if forced:
+        assert m == 0
+    elif name == "longest_segment":
         assert m == 64
     elif name != "three_groups_per_unit":
         assert m > 1
+    group = w.num_heads // w.num_kv_heads
+    if m == 0:
+        plan = _split_plan(wd, kernel)
+        per_item = plan.kv_heads_per_item
+        pieces = SP.even_shares_pieces(lens, partition_size=P, max_num_partitions=w.max_num_partitions,
+                                       max_ctx=w.block_tables.shape[1] * w.block_size,
+                                       num_kv_heads=w.num_kv_heads // per_item, groups=plan.work_groups,
+                                       cus=plan.compute_units)
     for s, n in enumerate(lens):
-        want = [j * m for j in range(-(-n // (m * P)))]
         for h in (0, w.num_heads - 1):
+            if m == 0:
+                want = [first for first, _, _ in pieces.get((s, h // (group * per_item)), [])]
+            else:
+                want = [j * m for j in range(-(-n // (m * P)))]
             assert (~torch.isnan(es[s, h])).nonzero().flatten().tolist() == want, (s, h)
+            # every slot a piece covers beyond its first holds the mark, in max_logits only
+            live = -(-n // P)
+            covered = [q for q in range(live) if q not in want]
+            assert all(_segment_mark(ml[s, h, q]) == m for q in covered), (s, h)
 
 
 @pytest.mark.parametrize("shape", ["few_items", "one_group_per_unit", "all_groups", "gqa"])

@@ -21,15 +21,66 @@ spec.loader.exec_module(mk)
 
 
 def test_device_choice_equals_the_host_restatement():
+    """The segment length the attention kernels choose and the slots in which they leave partials,
+    against the host restatement, on batches the fixture does not hold; and the same batches cut into
+    even shares on request."""
     dev = torch.device("cuda:0")
     checked = 0
     for case in mk.batches(seed=7, per_shape=6):
-        m, plan = mk.device_choice(case, dev)
-        if m is None:
+        m, plan, slots = mk.device_choice(case, dev)
+        if plan["form"] != _cabi.FA_SPLIT_FORM_SEGMENT:
             continue
-        assert mk.replay(case, plan) == m, (case, plan, m)
+        want = mk.replay(case, plan)
+        if m is not None:  # some piece covers two partitions, so the marks tell the cut
+            assert m == want, (case, plan, m, want)
+        assert slots == mk.replay_slots(case, plan, want), (case, plan, want)
+        m, plan, slots = mk.device_choice(case, dev, segment_partitions=-1)
+        assert m in (0, None) and slots == mk.replay_slots(case, plan, 0), (case, plan)
         checked += 1
-    assert checked >= 25
+    assert checked >= 25, checked
+
+
+def test_even_shares_on_request(oracle):
+    """options->segment_partitions = -1 cuts any batch into even shares: the rows' partitions laid end
+    to end, one contiguous run per work-group.  A small ragged batch (more work-groups than
+    partitions: shares of one partition or none), against the oracle and the restated cuts."""
+    dev = torch.device("cuda:0")
+    case = dict(head_size=128, num_kv_heads=4, group=2, fp8=False, token_major=False, block_size=16, partition_size=512,
+                lens=[5000, 0, 513, 1, 2100, 30000])
+    m, plan, slots = mk.device_choice(case, dev, segment_partitions=-1)
+    assert m in (0, None) and slots == mk.replay_slots(case, plan, 0)
+    w_cpu = W.make_config(2, num_seqs=6, pool_blocks=4096, lens=case["lens"])
+    _, ref32 = call_oracle(oracle.attention_ref, w_cpu, want_f32=True)
+    w = w_cpu.to(dev)
+    for kernel_kw in (dict(segment_partitions=-1), dict()):
+        bufs = runner.alloc_buffers(w)
+        runner.run_workload(w, "reduce", bufs, **kernel_kw)
+        torch.cuda.synchronize()
+        live = w_cpu.context_lens > 0
+        torch.testing.assert_close(bufs.out.float().cpu()[live], ref32[live], atol=1e-2, rtol=1e-2)
+        assert (bufs.out.cpu()[~live] == 0).all()
+
+
+def test_even_shares_full_serving_mix(oracle):
+    """A serving mix cut into even shares (128 sequences, log-normal lengths, E5M2 pools, bf16 queries,
+    8 query heads per kv head, sinks): every output row against the oracle."""
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.exp(torch.randn(128, generator=gen) * 0.75 + 8.3).long().clamp(64, 32768)
+    lens[3] = 0
+    w_cpu = W.make_config(4, num_seqs=128, pool_blocks=int(sum(-(-int(n) // 16) for n in lens)) + 8, lens=lens.tolist())
+    w_cpu.sinks = torch.linspace(-1, 3, w_cpu.num_heads).to(w_cpu.query.dtype)
+    w = w_cpu.to(dev)
+    bufs = runner.alloc_buffers(w)
+    runner.run_workload(w, "fp8_reduce", bufs, segment_partitions=-1)
+    torch.cuda.synchronize()
+    bits = bufs.max_logits.view(torch.int32).cpu()
+    marks = bits[(bits & mk.MARK_MASK) == mk.MARK_BITS]
+    assert marks.numel() and set((marks & 0xFF).tolist()) == {0}, "this batch is meant to be cut into even shares"
+    _, ref32 = call_oracle(oracle.attention_ref, w_cpu, want_f32=True)
+    live = w_cpu.context_lens > 0
+    torch.testing.assert_close(bufs.out.float().cpu()[live], ref32[live], atol=1e-2, rtol=1e-2)
+    assert (bufs.out.cpu()[~live] == 0).all()
 
 
 @pytest.mark.parametrize("fp8", [False, True], ids=["fp16", "e5m2"])

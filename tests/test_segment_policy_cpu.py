@@ -1,6 +1,6 @@
 """The segment-length rule of the split path, replayed on the host (tests/_segment_policy.py follows
 csrc/paged_attention_segment_policy.h statement by statement) against the lengths an MI355X chose
-for 58 recorded batches (tests/golden/segment_policy_cases.json), and against what the rule is meant
+for 39 recorded batches (tests/golden/segment_policy_cases.json), and against what the rule is meant
 to guarantee.  Upstream has one partial per partition (paged_attention_policy_v2.hpp:28,50); the
 rule, and so these vectors, are this library's own."""
 import importlib.util
@@ -26,7 +26,7 @@ with open(os.path.join(HERE, "golden", "segment_policy_cases.json")) as f:
 def test_the_recorded_batches_are_the_generators():
     # the fixture holds what batches(seed=0) draws (those that ran in the segment form)
     drawn = {json.dumps(b, sort_keys=True) for b in mk.batches(seed=0)}
-    assert len(CASES) >= 50
+    assert len(CASES) >= 35
     for c in CASES:
         b = {k: v for k, v in c.items() if k not in ("plan", "partitions_per_segment")}
         assert json.dumps(b, sort_keys=True) in drawn
@@ -70,6 +70,40 @@ def test_known_choices():
     # rows apart with a large load per unit: four segments per unit, as fitted on such batches
     big = _args(rows_apart=True)
     assert P.partitions_per_segment([40 * 512] * 8, **big) == 3  # ten partitions per unit over four (2.5)
+
+
+def test_even_shares_cover_every_partition_once_and_are_even():
+    """Even shares (on request): every live partition of every row lies in exactly one piece, pieces of a
+    work-group are contiguous on the tape, and no work-group has many more keys than it aims at (a
+    stretch of many short rows holds fewer: every piece has a cost of its own)."""
+    rng = random.Random(4)
+    for _ in range(120):
+        S = rng.choice((1, 5, 40, 128, 256))
+        psize = rng.choice((64, 256, 512))
+        lens = [rng.choice((0, rng.randint(1, 64 * psize))) for _ in range(S)]
+        hk = rng.choice((1, 4, 8))
+        cus = 256
+        groups = rng.choice((7, cus, 2 * cus))
+        kw = dict(partition_size=psize, max_num_partitions=64, max_ctx=64 * psize, num_kv_heads=hk, groups=groups, cus=cus)
+        pieces = P.even_shares_pieces(lens, **kw)
+        _, parts = P.live_partitions(lens, psize, 64, 64 * psize)
+        keys = [0] * groups
+        for s, p in enumerate(parts):
+            for k in range(hk):
+                if p == 0:
+                    assert (s, k) not in pieces
+                    continue
+                covered = []
+                for first, count, g in pieces[(s, k)]:
+                    covered += list(range(first, first + count))
+                    keys[g] += min(lens[s], (first + count) * psize) - first * psize
+                assert covered == list(range(p)), (lens[s], pieces[(s, k)])
+        total = sum(keys)
+        if total >= 64 * psize * groups:  # enough for the rounding to partitions not to matter
+            share = [k / total * groups for k in keys]
+            weight = [1.08, 0.92] if groups == 2 * cus else [1.0, 1.0]
+            half = groups // 2 if groups == 2 * cus else groups
+            assert all(x < weight[g >= half] + 0.08 for g, x in enumerate(share)), (min(share), max(share))
 
 
 def test_properties_over_random_batches():
