@@ -42,7 +42,8 @@ stream_ordered  host cost of a small decode step: blocking `run` calls (upstream
              the asynchronous torch.library operators, and a HIP-graph replay of them
 kv_cache_write  the step before the path (scatter of new K/V rows into the pools with E5M2
              rounding): kernel time by the same events, read + written bytes against the
-             HBM peak, and its CPU oracle on a bounded sample
+             HBM peak, and its CPU oracle on a bounded sample; random slots, and under
+             kv_cache_write_prefill the slots a prefill writes (consecutive per sequence)
 """
 from __future__ import annotations
 
@@ -311,10 +312,13 @@ def _reference_perf_recipe(steps, torch, W, runner, dev):
     return legs
 
 
-def _time_kv_cache_write(steps, torch, dev, cpu_leg):
+def _time_kv_cache_write(steps, torch, dev, cpu_leg, prefill_shaped=False):
     """Prefill-sized batch of the KV-cache writer: 32768 new tokens x 8 kv heads x 128, fp16
-    rows into E5M2 head-major pools of 65536 16-token blocks, random free slots.  Six
-    source/pool sets rotate (1.6 GB between two uses of the same bytes)."""
+    rows into E5M2 head-major pools of 65536 16-token blocks.  Slots: random free ones (the worst
+    case: every 128-byte row of a kv head lands somewhere else), or, prefill_shaped, what a prefill
+    writes: 16 sequences of 2048 new tokens each, a sequence's tokens in consecutive slots of blocks
+    that lie anywhere in the pool.  Six source/pool sets rotate (1.6 GB between two uses of the same
+    bytes)."""
     from flash_attention_factory_amd.lib import kv_cache_write
     N, Hk, D, B, NB, R = 32768, 8, 128, 16, 65536, 6
     g = torch.Generator(device=dev).manual_seed(0)
@@ -322,7 +326,12 @@ def _time_kv_cache_write(steps, torch, dev, cpu_leg):
     vals = [torch.randn(N, Hk, D, generator=g, device=dev, dtype=torch.float16) for _ in range(R)]
     pools = [(torch.zeros((NB, Hk, B, D), dtype=torch.uint8, device=dev),
               torch.zeros((NB, Hk, B, D), dtype=torch.uint8, device=dev)) for _ in range(R)]
-    slots = [torch.randperm(NB * B, generator=g, device=dev)[:N].to(torch.int64) for _ in range(R)]
+    if prefill_shaped:
+        within = torch.arange(N, device=dev) % B
+        slots = [torch.randperm(NB, generator=g, device=dev)[:N // B].repeat_interleave(B).to(torch.int64) * B + within
+                 for _ in range(R)]
+    else:
+        slots = [torch.randperm(NB * B, generator=g, device=dev)[:N].to(torch.int64) for _ in range(R)]
     view = lambda t: t.permute(0, 2, 1, 3).view(torch.float8_e5m2)
     ts = []
     for it in range(5 + steps):
@@ -333,7 +342,8 @@ def _time_kv_cache_write(steps, torch, dev, cpu_leg):
     us = float(torch.tensor(ts, dtype=torch.float64).mean())
     read_b, write_b = 2 * N * Hk * D * 2 + 8 * N, 2 * N * Hk * D
     res = dict(workload=f"kv_cache_write: {N} tokens x {Hk} kv heads x {D}, fp16 -> E5M2, head-major pool of "
-                        f"{NB} blocks of {B}, random slots",
+                        f"{NB} blocks of {B}, " + ("consecutive slots per sequence (16 sequences of 2048 tokens, blocks "
+                                                   "anywhere)" if prefill_shaped else "random slots"),
                kernel="kv_cache_write_kernel<F16, e5m2>", steps=steps, us_per_call=us,
                read_bytes=read_b, write_bytes=write_b, gbps_kernels=(read_b + write_b) / us / 1e3,
                hbm_frac=(read_b + write_b) / us / 1e3 / HBM_PEAK_GBPS)
@@ -676,6 +686,7 @@ def main():
         del built
         torch.cuda.empty_cache()
         line["kv_cache_write"] = _time_kv_cache_write(max(20, args.steps // 2), torch, dev, not args.no_cpu_baseline)
+        line["kv_cache_write_prefill"] = _time_kv_cache_write(max(20, args.steps // 2), torch, dev, False, prefill_shaped=True)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(1, torch, W)
         line["cpu_baseline"]["torch_reference"] = _torch_reference_baseline(torch, W)
@@ -699,6 +710,9 @@ def main():
     summary = [_summary_of("config1: " + args.layout, main_res["us_per_call"], line["roofline"])]
     for r in others:
         summary.append(_summary_of(r["workload"], r["us_per_call"], r["roofline"], r.get("kernel_us_mean")))
+    for key in ("kv_cache_write", "kv_cache_write_prefill"):
+        if key in line:
+            summary.append(dict(w=key, us=round(line[key]["us_per_call"], 2), frac=round(line[key]["hbm_frac"], 4)))
     for r in line.get("reference_perf_recipe", []):
         if r.get("form") is None or "forced" not in r["form"]:
             summary.append(dict(w=("recipe_e5m2_" if "E5M2" in r["workload"] else "recipe_fp16_") + r["kernel"],

@@ -13,7 +13,9 @@
 // and the slot one shift.  One work-group per token group, nothing looped or unrolled:
 // measured, a resident grid striding over tokens with 1, 2 or 4 tokens in flight per
 // thread is 3-18 % slower -- a read stream mixed with a write stream wants less in flight,
-// not more.
+// not more.  Nor is it the scatter that bounds the kernel: with the slots a prefill writes
+// (consecutive per sequence), and with the threads laid out so that those rows go out as runs of
+// 2 KiB per kv head, it takes the same 44-45 us as with random slots (built, verified, timed, not kept).
 #pragma once
 
 #include <type_traits>

@@ -62,6 +62,11 @@ inline int64_t loop_rows_of(const fa_paged_attention_shape &shape, const Resolve
   return (int64_t)shape.num_seqs * heads;
 }
 
+#ifndef FA_STRICT_HEADS
+#define FA_STRICT_HEADS 4
+#endif
+constexpr int kStrictHeads = FA_STRICT_HEADS;
+
 enum SplitForm { kSplitFormGrid = 0, kSplitFormSegment = 1, kSplitFormLoop = 2 };  // = fa_split_form
 
 // compute_units: of the GPU the call would run on
@@ -104,9 +109,17 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float attention_us = 0.f;
-  const bool segment_form = SegmentSplit<KV8>::use && r.schedule == FA_SCHEDULE_AUTO && shape.num_seqs <= kSegmentMaxSeqs &&
-                            shape.num_pool_blocks > 0 && r.partition_size < kSegmentMaxContext &&
-                            (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
+  const bool persistent_fits = SegmentSplit<KV8>::use && shape.num_seqs <= kSegmentMaxSeqs && shape.num_pool_blocks > 0 &&
+                               r.partition_size < kSegmentMaxContext &&
+                               (int64_t)shape.max_blocks_per_seq * shape.block_size < kSegmentMaxContext;
+  const bool segment_form = persistent_fits && r.schedule == FA_SCHEDULE_AUTO;
+  // Upstream's decomposition -- one partial per partition, every live slot of the scratch arrays
+  // written as upstream writes it -- by resident work-groups: each wavefront takes one kv head of four
+  // adjacent ones and walks whole partitions of it, its loads running on across the partitions'
+  // ends; a partial goes from its registers to tmp_out, no LDS, nobody waited for.  (One work-group per
+  // partition, the form below, starts its stream anew for every 512 keys.)
+  const bool strict_form = persistent_fits && r.schedule == FA_SCHEDULE_GRID && !ext && !r.pair_heads &&
+                           p.num_kv_heads % 4 == 0;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
   // columns, or in the segment form two tiles of 16 held by every wavefront.
   // Every launch fills its own rows of the scratch arrays, the reduce kernel runs once.
@@ -116,7 +129,22 @@ inline fa_status launch_paged_attn_v2_batch(void *out, const void *query, const 
   for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {
     p.query_first = q0;
     p.query_count = std::min(per_launch, r.query_len - q0);
-    if (segment_form) {
+    if (strict_form) {
+      constexpr int SW = SegmentSplit<KV8>::waves;
+      static_assert(SW == 4, "four kv heads per work-group, one wavefront each");
+      auto kernel = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ, Pipeline<KV8>::tiles_per_chunk, false, kStrictHeads>;
+      int resident = 0, cus = 0;
+      FA_HIP_CHECK(resident_groups(kernel, SW * 64, &resident, &cus));
+      p.compute_units = cus;
+      p.segment_force = 1;  // one partial per partition
+      const int64_t max_items = (int64_t)shape.num_seqs * shape.max_num_partitions * (p.num_kv_heads / kStrictHeads);
+      if (r.plan) {
+        r.plan->work_groups = (int)std::min<int64_t>(resident, max_items);
+        r.plan->kv_heads_per_item = kStrictHeads;
+        return FA_OK;
+      }
+      FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)std::min<int64_t>(resident, max_items)), dim3(SW * 64), 0, p));
+    } else if (segment_form) {
       // Segment form: multi-wavefront work-groups, one partial per segment of partitions.
       constexpr int SW = SegmentSplit<KV8>::waves;
       auto plain = paged_attn_segment_kernel<HEAD_SIZE, QT, KVF, SW, SegmentSplit<KV8>::occ,

@@ -38,6 +38,12 @@
 #include "paged_attention_loop_persistent_kernel.h"
 #include "paged_attention_segment_policy.h"
 
+// Builds that time what the stores of the partials cost (profiles/): 1 leaves out the rows of tmp_out,
+// 2 the scalars as well.  Their results are wrong; the product is built with 0.
+#ifndef FA_COST_PROBE
+#define FA_COST_PROBE 0
+#endif
+
 namespace fa {
 
 //
@@ -55,8 +61,10 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
   constexpr int NR = W::NR;
   constexpr int NDT = W::NDT;
   constexpr int SL = NR / NT;
-  static_assert(NT > 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 4 && SL % 4 == 0,
+  static_assert(NT >= 1 && NW % HPW == 0 && NR % NT == 0 && SL >= 4 && SL % 4 == 0,
                 "each wavefront stores whole 16-byte pieces");
+  // NT == 1: every wavefront has a kv head of its own and the whole of each item's chunks, so an item's
+  // state never leaves its registers: no LDS, no waiting for the others.
 
   FA_TIMELINE_STAMP(0);
   FA_TIMELINE_WHERE();
@@ -117,10 +125,58 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     if (lane == 0)
       __hip_atomic_fetch_add(&sm_arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
+  // Store this wavefront's slice o[SL] of an item's merged, un-normalised output (maximum M in base-2
+  // units, sum L) as the item's partial -- or, where the item is its row's only piece, as the row's result.
+  auto store_slice = [&](const Item &it, float M, float L, const float (&o)[SL], float out_mul) {
+    if (wa.col_valid && wa.keeps_output()) {
+      const int head = it.kvh * p.group + wa.col_g;
+      int64_t row = it.seq;
+      float inv = p.out_scale / L;
+      if constexpr (EXT) {
+        row = (int64_t)it.seq * p.query_len + wa.col_q;
+        inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key of the segment
+      }
+      const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
+      const int d0 = wa.out_elem(4 * r * NDT + tw * SL);
+      // the row's only partial is its result (PagedAttnParams::final_out); it.ctx is the length as
+      // far as the scratch arrays hold it
+      if (p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx)
+        W::template store_q<SL>(
+            reinterpret_cast<char *>(p.final_out) + ((row * p.num_heads + head) * wa.out_row_elems() + d0) * 2, o, inv);
+      else if (FA_COST_PROBE < 1)  // (cost probes: 1 = no rows of partials, 2 = no scalars either)
+        W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
+      if ((wa.paired() ? (r & 1) == 0 : r == 0) && tw == 0 && FA_COST_PROBE < 2) {  // one lane per column, see merge_and_store
+        p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
+        p.exp_sums[slot] = L;
+      }
+    }
+    // the slots that the piece covers beyond its first tell the reduce kernel that they hold no partial
+    if (tw == 0 && it.parts > 1) {
+      const int rows = EXT ? p.query_count : 1;  // query tokens of the launch
+      for (int q = 0; q < rows; ++q) {
+        const int64_t row = EXT ? (int64_t)it.seq * p.query_len + p.query_first + q : it.seq;
+        mark_covered_slots(p.max_logits, (row * p.num_heads + (int64_t)it.kvh * p.group) * p.max_num_partitions + it.part0,
+                           p.group, p.max_num_partitions, it.parts, lane, items.m);
+      }
+    }
+  };
+  // NT == 1: the item at hand straight from the registers.  (A lane holds NR consecutive floats of its
+  // head's row, so a store instruction puts 16 bytes into each of 32 lines.  Exchanging pieces through
+  // LDS first, so that eight lanes write a whole line, was built and timed: 317 -> 310 us on the serving
+  // mix with one partial per partition, 120 -> 140 us on the long-context batch; not kept.)
+  auto store_own = [&](const Item &it, float out_mul) {
+    wa.settle();
+    const float L = rows_sum(wa.l);
+    float o[SL];
+#pragma unroll
+    for (int e = 0; e < SL; ++e) o[e] = wa.acc_at(e);
+    store_slice(it, wa.m, L, o, out_mul);
+  };
   // Merge the NW published states of the work-group's n-th item, normalise, store this
   // wavefront's slice of the partial (see the persistent loop kernel for why the wait
   // always ends and why a buffer is never overwritten while it is read).
   auto finish = [&](int n, const Item &it, float out_mul) {
+    if constexpr (NT > 1) {  // (NT == 1: stored when the item ended, store_own)
     const int b = n & 1;
     const int target = NW * ((n >> 1) + 1);
     bool arrived = false;
@@ -156,36 +212,7 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
       for (int u = 0; u < NT; ++u) a += f[u] * sm_acc[b][w0 + u][tw * SL + e][lane];
       o[e] = a;
     }
-    if (wa.col_valid && wa.keeps_output()) {
-      const int head = it.kvh * p.group + wa.col_g;
-      int64_t row = it.seq;
-      float inv = p.out_scale / L;
-      if constexpr (EXT) {
-        row = (int64_t)it.seq * p.query_len + wa.col_q;
-        inv = L > 0.f ? out_mul / L : 0.f;  // L = 0: the query token sees no key of the segment
-      }
-      const int64_t slot = (row * p.num_heads + head) * p.max_num_partitions + it.part0;
-      const int d0 = wa.out_elem(4 * r * NDT + tw * SL);
-      // the row's only partial is its result (PagedAttnParams::final_out); it.ctx is the length as
-      // far as the scratch arrays hold it
-      if (p.final_out != nullptr && it.part0 == 0 && it.tok_end >= it.ctx)
-        W::template store_q<SL>(
-            reinterpret_cast<char *>(p.final_out) + ((row * p.num_heads + head) * wa.out_row_elems() + d0) * 2, o, inv);
-      else
-        W::template store_f32<SL>(reinterpret_cast<float *>(p.out) + slot * wa.out_row_elems() + d0, o, inv);
-      if ((wa.paired() ? (r & 1) == 0 : r == 0) && tw == 0) {  // one lane per column, see merge_and_store
-        p.max_logits[slot] = M * kLn2;  // natural-log units, as upstream stores them
-        p.exp_sums[slot] = L;
-      }
-    }
-    // the slots that the piece covers beyond its first tell the reduce kernel that they hold no partial
-    if (tw == 0 && it.parts > 1) {
-      const int rows = EXT ? p.query_count : 1;  // query tokens of the launch
-      for (int q = 0; q < rows; ++q) {
-        const int64_t row = EXT ? (int64_t)it.seq * p.query_len + p.query_first + q : it.seq;
-        mark_covered_slots(p.max_logits, (row * p.num_heads + (int64_t)it.kvh * p.group) * p.max_num_partitions + it.part0,
-                           p.group, p.max_num_partitions, it.parts, lane, items.m);
-      }
+    store_slice(it, M, L, o, out_mul);
     }
   };
 
@@ -285,7 +312,8 @@ paged_attn_segment_kernel(const PagedAttnParams p) {
     }
     if (!has_next) FA_TIMELINE_STAMP(3);
     if (owed) finish(n - 1, prev, prev_out_mul);
-    publish(n);
+    if constexpr (NT == 1) store_own(cur, EXT ? cur_ext.out_mul : 1.f);
+    else publish(n);
 
     if (!has_next) break;
     prev = cur;
