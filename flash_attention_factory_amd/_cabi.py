@@ -38,6 +38,7 @@ EXPORTS = (
     "fa_paged_attention_reduce_static_scratch",
     "fa_paged_attention_kernel_status",
     "fa_paged_attention_reduce_plan",
+    "fa_paged_attention_init",
 )
 
 ABI_REVISION = 8
@@ -217,6 +218,8 @@ def load() -> ctypes.CDLL:
     L.fa_paged_attention_reduce_plan.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(Options), ctypes.c_int32,
                                                  ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(SplitPlan)]
     L.fa_paged_attention_reduce_plan.restype = ctypes.c_int32
+    L.fa_paged_attention_init.argtypes = []
+    L.fa_paged_attention_init.restype = ctypes.c_int32
     L.fa_paged_attention_kernel_status.argtypes = [P, ctypes.c_int32]
     L.fa_paged_attention_kernel_status.restype = ctypes.c_int32
     if L.fa_paged_attention_abi_version() != ABI_REVISION:
@@ -224,6 +227,12 @@ def load() -> ctypes.CDLL:
                            f"written for {ABI_REVISION}: rebuild the library")
     _lib = L
     return L
+
+
+def init() -> None:
+    """What the library sets up once per GPU, now, on the current device (fa_paged_attention_init): to be
+    called outside a HIP graph capture before calls are recorded into one."""
+    check(load().fa_paged_attention_init())
 
 
 def kernel_status(stream: int = 0, clear: bool = True) -> None:

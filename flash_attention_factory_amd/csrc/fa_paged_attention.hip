@@ -161,6 +161,19 @@ FA_EXPORT int32_t fa_kv_cache_write(const void *key, const void *value, void *ke
   return fa::launch_kv_cache_write(key, value, key_cache, value_cache, slot_mapping, &sh, c.options());
 }
 
+FA_EXPORT int32_t fa_paged_attention_init(void) {
+  fa::error_buffer()[0] = 0;
+  int32_t *word = nullptr;
+  fa_status st = fa::kernel_status_of_current_device(&word);
+  if (st != FA_OK) return st;
+  unsigned char *base = nullptr;
+  st = static_scratch_of_current_device(&base);
+  if (st != FA_OK) return st;
+  int cus = 0;
+  FA_HIP_CHECK(fa::compute_units_of_current_device(&cus));
+  return FA_OK;
+}
+
 FA_EXPORT int32_t fa_paged_attention_reduce_plan(const fa_paged_attention_shape *shape,
                                                  const fa_paged_attention_options *options, int32_t max_context_len,
                                                  int32_t kv_fp8, int32_t compute_units, fa_split_plan *plan) {

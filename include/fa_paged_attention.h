@@ -230,6 +230,10 @@ int32_t fa_paged_attention_reduce(void *out, const void *query, const void *key_
  * live in a fixed array of FA_STATIC_SCRATCH_BYTES that the library holds in device memory on
  * every GPU it runs on until the process ends.  The call allocates nothing, on the host or on the
  * device, and frees nothing.
+ * The array is part of the library's code object: every process that loads the library holds
+ * FA_STATIC_SCRATCH_BYTES of device memory on every GPU it touches, whether or not this entry point
+ * is ever called.  Under HIP graph capture: fa_paged_attention_init() and one eager call of the same
+ * shape first (see there).
  *   needs  2 * align256(4 * slots) + 4 * slots * head_size bytes,
  *          slots = num_seqs * max(query_len, 1) * num_heads * max_num_partitions;
  *          more than FA_STATIC_SCRATCH_BYTES -> FA_ERR_SCRATCH_TOO_SMALL, nothing is launched
@@ -261,6 +265,15 @@ int32_t fa_paged_attention_fp8_reduce(void *out, const void *query, const void *
                                       float *max_logits, float *tmp_out,
                                       const fa_paged_attention_shape *shape,
                                       const fa_paged_attention_options *options);
+
+/* Everything the library sets up once per GPU, done now on the current device instead of inside the
+ * first call there: the device addresses of its two static device arrays (the status word of
+ * fa_paged_attention_kernel_status and the scratch of fa_paged_attention_reduce_static_scratch, both
+ * through hipGetSymbolAddress, which may load the code object) and the device's compute-unit count.
+ * A caller that records calls into a HIP graph calls this first, outside the capture, and makes one
+ * eager call of each shape it will record (the first launch of a kernel instance asks the occupancy
+ * calculator how many of its work-groups stay resident).  No counterpart upstream. */
+int32_t fa_paged_attention_init(void);
 
 /* Text of the last failure on the calling thread ("" if none). */
 const char *fa_last_error(void);
