@@ -26,6 +26,10 @@ configs      the other four configurations, each timed the same way, each with a
              leg: upstream's decomposition, one partial per 512-token partition
 lds_staging  the FP8 configurations in the grid form, K/V through registers against K/V staged
              through LDS by direct-to-LDS loads
+single_head_groups  the two configurations with one query head per kv head (1 and 3) by lane dot
+             products and fp32 multiply-adds in the VALU (schedules FA_SCHEDULE_GRID_VALU, FA_SCHEDULE_VALU)
+             against the matrix cores (15 of 16 MFMA columns idle): the grid form of both, and the
+             resident form beside the configurations' own figures above
 reference_perf_recipe  the shape upstream's own perf loop runs (test_paged.py:607-631 and the FP8
              twin: 64 sequences of 1500 tokens, 64 or 40 query heads over 8 kv heads, head size 64,
              block size 64, sinks, its token-major pools) through the loop and the split kernels,
@@ -680,6 +684,17 @@ def main():
                 _, r = _time_config(built[idx], sub_steps, args.warmup, torch, W, runner, dev, schedule=schedule)
                 line["lds_staging"].append(dict(workload=r["workload"], schedule=name, kernel_us_mean=r["kernel_us_mean"],
                                                 us_per_call=r["us_per_call"], hbm_frac=r["hbm_frac"]))
+        # query groups of one head: the grid form by the matrix cores (schedule 1) against the grid
+        # form by dot products in the VALU (schedule 4), beside the persistent forms timed above
+        line["single_head_groups"] = []
+        for idx in (1, 3):
+            if idx not in built:
+                continue
+            for schedule, name in ((1, "grid form, matrix cores"), (4, "grid form, VALU dot products"),
+                                   (5, "resident work-groups, VALU dot products")):
+                _, r = _time_config(built[idx], sub_steps, args.warmup, torch, W, runner, dev, schedule=schedule)
+                line["single_head_groups"].append(dict(workload=r["workload"], schedule=name, kernel_us_mean=r["kernel_us_mean"],
+                                                       us_per_call=r["us_per_call"], hbm_frac=r["hbm_frac"]))
         line["reference_perf_recipe"] = _reference_perf_recipe(max(20, args.steps // 2), torch, W, runner, dev)
         line["stream_ordered"] = _time_stream_ordered(max(200, args.steps), torch, W, runner, dev)
     if not args.no_kv_cache_write:

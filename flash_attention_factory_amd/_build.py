@@ -16,16 +16,23 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
+def build(verbose: bool = False, extra_flags=(), output: str = LIBRARY) -> str:
+    """The product library, or with extra_flags and another output a debug build beside it
+    (-DFA_TIMELINE: in-kernel timeline; -DFA_COST_PROBE=1|2: the segment kernels without their stores
+    of partials), which FA_PAGED_ATTENTION_LIBRARY selects at run time."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, SOURCE, "-o", LIBRARY]
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, SOURCE, "-o", output]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
-    return LIBRARY
+    return output
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    import argparse
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--output", default=LIBRARY)
+    args, flags = ap.parse_known_args()  # everything else goes to hipcc (-DFA_TIMELINE ...)
+    print(build(verbose=True, extra_flags=flags, output=os.path.abspath(args.output)))

@@ -9,7 +9,9 @@ import ctypes
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIBRARY = os.path.join(_PKG, "libfa_paged_attention.so")
+# FA_PAGED_ATTENTION_LIBRARY names another build of the same sources (a debug build with the in-kernel
+# timeline or a cost probe compiled in); there is no fallback to anything that is not this library
+LIBRARY = os.path.abspath(os.environ.get("FA_PAGED_ATTENTION_LIBRARY") or os.path.join(_PKG, "libfa_paged_attention.so"))
 
 FA_OK = 0
 FA_ERR_NULL_POINTER = 1
@@ -58,6 +60,8 @@ FA_SCHEDULE_AUTO = 0
 FA_SCHEDULE_GRID = 1
 FA_SCHEDULE_GRID_LDS = 2
 FA_SCHEDULE_SPLIT = 3
+FA_SCHEDULE_GRID_VALU = 4
+FA_SCHEDULE_VALU = 5
 
 FA_SPLIT_FORM_GRID = 0
 FA_SPLIT_FORM_SEGMENT = 1

@@ -27,6 +27,7 @@
 #include "paged_attention_policy.h"
 #include "paged_attention_reduce_kernel.h"
 #include "paged_attention_segment_kernel.h"
+#include "paged_attention_valu_kernel.h"
 
 namespace fa {
 
@@ -264,8 +265,9 @@ inline fa_status validate_and_resolve(const void *out, const void *query, const 
   }
   r->schedule = o ? o->schedule : FA_SCHEDULE_AUTO;
   if (r->schedule != FA_SCHEDULE_AUTO && r->schedule != FA_SCHEDULE_GRID && r->schedule != FA_SCHEDULE_GRID_LDS &&
-      r->schedule != FA_SCHEDULE_SPLIT)
-    return fail(FA_ERR_BAD_SHAPE, "schedule %d is none of auto (0), grid (1), grid with LDS staging (2), split (3)",
+      r->schedule != FA_SCHEDULE_SPLIT && r->schedule != FA_SCHEDULE_GRID_VALU && r->schedule != FA_SCHEDULE_VALU)
+    return fail(FA_ERR_BAD_SHAPE,
+                "schedule %d is none of auto (0), grid (1), grid with LDS staging (2), split (3), without matrix cores: grid (4), persistent (5)",
                 r->schedule);
   r->keep_split = r->schedule == FA_SCHEDULE_SPLIT;  // otherwise the library's own choice
   if (r->keep_split) r->schedule = FA_SCHEDULE_AUTO;

@@ -11,6 +11,25 @@
 
 #include "launch_common.h"
 
+// Persistent dot-product kernel: wavefronts per work-group, and a cap on work-groups per compute unit
+// (0: as many as stay resident).  Measured on the two single-head benchmark batches (16-bit / E5M2 cache,
+// us): four wavefronts and every resident work-group (three or four per unit) 104.6 / 59.5, eight
+// wavefronts 104.6 / 56.4, four wavefronts and two work-groups per unit 102.4 / 56.4 -- and 101.6 / 55.3
+// for the matrix-core kernel of the same schedule, which therefore stays the library's choice.
+#ifndef FA_VALU_WAVES
+#define FA_VALU_WAVES 4
+#endif
+// wavefronts per SIMD its registers are held to: a 16-bit cache keeps twice the bytes of a chunk in registers
+#ifndef FA_VALU_OCC_16
+#define FA_VALU_OCC_16 3
+#endif
+#ifndef FA_VALU_OCC_FP8
+#define FA_VALU_OCC_FP8 4
+#endif
+#ifndef FA_VALU_GROUPS_PER_UNIT
+#define FA_VALU_GROUPS_PER_UNIT 2
+#endif
+
 namespace fa {
 
 // The launches of one batch that a single kernel launch can take: persistent form for up to
@@ -33,7 +52,9 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
   // score modifiers, several query tokens, per-head or per-block scales: the extended instances
   const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
   float total_us = 0.f;
-  const bool persistent = kUsePersistentLoop && r.schedule == FA_SCHEDULE_AUTO &&
+  // lane dot products instead of the matrix cores (paged_attention_valu_kernel.h): groups of one head
+  const bool dot_fits = HEAD_SIZE == 128 && std::is_same<QT, F16>::value && p.group == 1 && !ext && !r.pair_heads;
+  const bool persistent = kUsePersistentLoop && (r.schedule == FA_SCHEDULE_AUTO || (r.schedule == FA_SCHEDULE_VALU && dot_fits)) &&
                           shape.num_seqs <= kLoopPersistentMaxSeqs && shape.num_pool_blocks > 0 &&
                           max_ctx < kLoopPersistentMaxContext;
   // One launch per group of query tokens that fit the MFMA columns (one launch for decode): 16
@@ -43,7 +64,16 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
   for (int q0 = 0; q0 < r.query_len; q0 += per_launch) {
     p.query_first = q0;
     p.query_count = std::min(per_launch, r.query_len - q0);
-    if (persistent) {
+    if (persistent && r.schedule == FA_SCHEDULE_VALU) {
+      if constexpr (HEAD_SIZE == 128 && std::is_same<QT, F16>::value) {
+        constexpr int VW = FA_VALU_WAVES;
+        auto kernel = paged_attn_valu_persistent_kernel<KVF, VW, Pipeline<KV8>::stream_loads_loop, (KV8 ? FA_VALU_OCC_FP8 : FA_VALU_OCC_16)>;
+        int resident = 0, cus = 0;
+        FA_HIP_CHECK(resident_groups(kernel, VW * 64, &resident, &cus));
+        if (FA_VALU_GROUPS_PER_UNIT > 0) resident = std::min(resident, FA_VALU_GROUPS_PER_UNIT * cus);
+        FA_HIP_CHECK(timer.launch(kernel, dim3((unsigned)std::min<int64_t>(resident, items)), dim3(VW * 64), 0, p));
+      }
+    } else if (persistent) {
       // Persistent form: resident work-groups walk the (sequence, kv head) items, longest
       // sequences first, with the next item's first loads issued before each merge.
       constexpr int PW = PersistentLoop<KV8>::waves;
@@ -90,6 +120,12 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
       if constexpr (KV8 && HEAD_SIZE == 128) {
         const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);
         FA_HIP_CHECK(timer.launch(paged_attn_lds_kernel<HEAD_SIZE, QT, KVF, false, 8, 2>, grid, dim3(8 * 64), 0, p));
+      }
+    } else if (dot_fits && r.schedule == FA_SCHEDULE_GRID_VALU) {
+      // grid form without the matrix cores: lane dot products, for query groups of one head
+      if constexpr (HEAD_SIZE == 128 && std::is_same<QT, F16>::value) {
+        const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);
+        FA_HIP_CHECK(timer.launch(paged_attn_valu_kernel<KVF, NW, Pipeline<KV8>::stream_loads_loop>, grid, dim3(NW * 64), 0, p));
       }
     } else if (ext) {
       const dim3 grid(p.num_kv_heads, 1, shape.num_seqs);

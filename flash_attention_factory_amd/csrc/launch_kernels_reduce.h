@@ -22,14 +22,15 @@ namespace fa {
 // second kernel costs 4-5 us of every call whatever it finds to do, and a row of a thousand keys is
 // read by one work-group in little more than that.  What the host knows of a batch without reading
 // device memory is an upper bound on its rows: max_context_len (upstream passes seqlen_k), the block
-// table's width and the scratch arrays' capacity.  Measured over 150 batches (head sizes 64 and 128,
+// table's width and the scratch arrays' capacity.  Measured over 113 batches (head sizes 64 and 128,
 // 16-bit and byte caches, 2 to 128 sequences of up to 4096 keys, equal and ragged lengths), the loop
-// kernel against the split kernels at their best segment length:
-//   rows of at most kSplitNeverBelowTokens keys        the loop kernel is as fast or faster in every
-//                                                      batch (1.0-1.9 times)
-//   rows of at most kSplitFullGpuBelowTokens keys,     faster in 26 of 30 batches (by 2-21 %; slower
+// kernel against the split kernels:
+//   rows of at most kSplitNeverBelowTokens keys        the loop kernel is as fast or faster in all 33
+//                                                      batches (1.0-1.9 times)
+//   rows of at most kSplitFullGpuBelowTokens keys,     faster in 16 of 18 batches (by 2-18 %; slower
 //   and a (sequence, kv head) row for every unit       by 6 and 18 % in two ragged ones)
-//   anything longer, or fewer rows                     the split kernels win, up to 2.7 times
+//   anything longer, or fewer rows                     the split kernels win in 45 of 62 batches, up
+//                                                      to 2.7 times (the loop kernel by at most 20 %)
 // In the first two cases the call IS the loop kernel: one launch, the same `out`, the scratch
 // arrays untouched, and {t, 0} as its two times.
 constexpr int kSplitNeverBelowTokens = 1024;

@@ -116,9 +116,16 @@ typedef enum fa_mask { FA_MASK_ALIBI = 1, FA_MASK_SOFTCAP = 2, FA_MASK_WINDOW = 
  * anything else falls back to FA_SCHEDULE_GRID).  FA_SCHEDULE_SPLIT is FA_SCHEDULE_AUTO except that a
  * reduce entry always runs its two kernels, also where rows are so short that FA_SCHEDULE_AUTO runs the
  * single-pass kernel instead (fa_paged_attention_reduce_plan); loop entries take it as FA_SCHEDULE_AUTO.
- * `out` is the same under all four. */
+ * FA_SCHEDULE_GRID_VALU and FA_SCHEDULE_VALU are the loop entries without the matrix cores: lane dot
+ * products and fp32 multiply-adds, for query groups of ONE head (head size 128, fp16 queries, no score
+ * modifiers or query tokens; anything else, and the reduce entries, run as FA_SCHEDULE_GRID) -- the first
+ * in the grid form, the second as resident work-groups like FA_SCHEDULE_AUTO.  They are there to be
+ * measured beside the matrix-core kernels, which the other schedules use for every group size and
+ * which are as fast or faster in the resident form.
+ * `out` is the same under all of them, to the tolerance of the path. */
 typedef enum fa_schedule {
-  FA_SCHEDULE_AUTO = 0, FA_SCHEDULE_GRID = 1, FA_SCHEDULE_GRID_LDS = 2, FA_SCHEDULE_SPLIT = 3
+  FA_SCHEDULE_AUTO = 0, FA_SCHEDULE_GRID = 1, FA_SCHEDULE_GRID_LDS = 2, FA_SCHEDULE_SPLIT = 3,
+  FA_SCHEDULE_GRID_VALU = 4, FA_SCHEDULE_VALU = 5
 } fa_schedule;
 
 typedef enum fa_kv_scale { FA_KV_SCALE_TENSOR = 0, FA_KV_SCALE_HEAD = 1, FA_KV_SCALE_BLOCK = 2 } fa_kv_scale;

@@ -311,9 +311,9 @@ def test_kv_scale_argument_checks(L):
 def test_schedule_values(L):
     for split in (False, True):
         for fp8 in (False, True):
-            for schedule in (0, 1, 2, 3):  # the LDS form falls back to the grid form where it does not apply
+            for schedule in (0, 1, 2, 3, 4, 5):  # the LDS and dot-product forms fall back to the grid form where they do not apply
                 assert _call(L, split=split, fp8=fp8, schedule=schedule)[0] == _cabi.FA_OK
-            code, text = _call(L, split=split, fp8=fp8, schedule=4)
+            code, text = _call(L, split=split, fp8=fp8, schedule=6)
             assert code == _cabi.FA_ERR_BAD_SHAPE and "schedule" in text
 
 

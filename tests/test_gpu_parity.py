@@ -10,7 +10,7 @@ import os
 import pytest
 import torch
 
-from flash_attention_factory_amd import workloads as W
+from flash_attention_factory_amd import _cabi, workloads as W
 from _torch_ref import call_oracle, out_pt_reference
 
 pytestmark = pytest.mark.gpu
@@ -161,6 +161,35 @@ def test_schedule_option(oracle, fp8, schedule):
                 torch.testing.assert_close(bufs.exp_sums[s, :, :live].cpu(), es[s, :, :live], atol=1e-4, rtol=1e-4)
                 torch.testing.assert_close(bufs.tmp_out[s, :, :live].cpu(), tmp[s, :, :live], atol=tmp_atol, rtol=1e-2)
                 assert torch.isnan(bufs.max_logits[s, :, live:]).all()
+
+
+@pytest.mark.parametrize("fp8", [False, True], ids=["kv16", "fp8"])
+def test_dot_product_kernel_for_single_head_groups(oracle, fp8):
+    """schedule = FA_SCHEDULE_GRID_VALU: the loop path for query groups of one head by lane dot products
+    and fp32 multiply-adds instead of the matrix cores.  Edge lengths around its 32-token chunks and the
+    rows of one load instruction, an empty sequence, sinks, both layouts, E4M3 bytes -- and the whole of
+    the benchmark configuration of its cache type."""
+    lens = [1, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 255, 256, 257, 700, 2048, 0]
+    cfg = 3 if fp8 else 1
+    variants = [dict(), dict(layout=W.TOKEN_MAJOR)] + ([dict(fp8_dtype=torch.float8_e4m3fn)] if fp8 else [])
+    for schedule in (_cabi.FA_SCHEDULE_GRID_VALU, _cabi.FA_SCHEDULE_VALU):  # grid form, persistent form
+        for kw in variants:
+            w = W.make_config(cfg, num_seqs=len(lens), pool_blocks=4096, lens=lens, **kw)
+            assert w.num_heads == w.num_kv_heads and w.head_size == 128
+            w.sinks = torch.linspace(-1, 2, w.num_heads).to(w.query.dtype)
+            bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)
+            _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/{kw}")
+        # few items of few chunks: work-groups with one item, wavefronts without a chunk of their own
+        w = W.make_config(cfg, num_seqs=3, pool_blocks=512, lens=[40, 0, 97])
+        bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)
+        _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/few")
+        w = W.make_config(cfg)
+        bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)
+        _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/full")
+        # a group of several heads is not these kernels': the call runs on the matrix cores
+        w = W.make_config(4 if fp8 else 2, num_seqs=3, pool_blocks=4096, lens=[700, 33, 1537])
+        bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)
+        _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/fallback")
 
 
 def test_lds_staged_kernel_full_size(oracle):
