@@ -186,6 +186,20 @@ inline fa_status launch_paged_attn_loop(void *out, const void *query, const void
   // most sequences one launch takes: what the persistent kernel ranks, or what the grid's third
   // dimension holds
   constexpr int kGridMaxSeqs = 65535;
+  // Batches beyond what one persistent launch ranks, 16-bit cache, one query head per kv head: the grid
+  // form by lane dot products (paged_attention_valu_kernel.h) beats both the sub-batches of persistent
+  // launches and the grid form on the matrix cores -- 512 sequences of the Llama-7B decode shape: 1681 us
+  // against 1712 and 1752, 200 sequences: 655 against 670 and 680.  (With a byte cache the two grid forms
+  // time the same, 808 against 817 us, and the matrix-core one stays.)
+  Resolved dot = r;
+  if constexpr (KVF == kKv16 && HEAD_SIZE == 128 && std::is_same<QT, F16>::value) {
+    const bool ext = r.mask_flags != 0 || r.query_len > 1 || r.kv_scale_mode != 0;
+    if (r.schedule == FA_SCHEDULE_AUTO && shape.num_seqs > kLoopPersistentMaxSeqs && shape.num_heads == shape.num_kv_heads &&
+        !ext && !r.pair_heads)
+      dot.schedule = FA_SCHEDULE_GRID_VALU;
+  }
+  if (dot.schedule != r.schedule) return launch_paged_attn_loop<HEAD_SIZE, QT, KVF>(out, query, key_cache, value_cache, block_tables,
+                                                                                    context_lens, scale, 0, shape, dot);
   const bool persistent_pieces = PersistentLoop<(KVF != kKv16)>::sub_batches && r.schedule == FA_SCHEDULE_AUTO &&
                                  loop_persistent_fits(shape) && shape.num_seqs > kLoopPersistentMaxSeqs;
   const int most = persistent_pieces ? kLoopPersistentMaxSeqs : kGridMaxSeqs;

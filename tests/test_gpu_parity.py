@@ -186,6 +186,15 @@ def test_dot_product_kernel_for_single_head_groups(oracle, fp8):
         w = W.make_config(cfg)
         bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)
         _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/full")
+        # more sequences than one resident launch lists (with a 16-bit cache the library's own choice is the grid
+        # form of these kernels then: schedule 0 below)
+        gen = torch.Generator().manual_seed(11)
+        many = [int(x) for x in torch.randint(0, 300, (150,), generator=gen)]
+        w = W.make_config(cfg, num_seqs=len(many), pool_blocks=4096, lens=many)
+        w.sinks = torch.linspace(-2, 1, w.num_heads).to(w.query.dtype)
+        for sched in (schedule, 0):
+            bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=sched)
+            _check(bufs.out, w, oracle, f"{w.name}/valu{sched}/150 sequences")
         # a group of several heads is not these kernels': the call runs on the matrix cores
         w = W.make_config(4 if fp8 else 2, num_seqs=3, pool_blocks=4096, lens=[700, 33, 1537])
         bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop", schedule=schedule)

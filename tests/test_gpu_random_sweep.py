@@ -162,7 +162,13 @@ def _run_case(oracle, c):
     alibi = okw["alibi_slopes"].to(dev) if "alibi_slopes" in okw else None
     kv, vv = (wd.key_cache.permute(0, 2, 1, 3), wd.value_cache.permute(0, 2, 1, 3)) if w.layout == W.HEAD_MAJOR \
         else (wd.key_cache, wd.value_cache)
-    for kernel in (("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")):
+    kernels = ("fp8_loop", "fp8_reduce") if fp8 else ("loop", "reduce")
+    if c.get("dot_schedules"):
+        # the loop kernels without the matrix cores (schedules FA_SCHEDULE_GRID_VALU, FA_SCHEDULE_VALU)
+        kernels = tuple((kernels[0], sched) for sched in c["dot_schedules"])
+    for kernel in kernels:
+        if isinstance(kernel, tuple):
+            kernel, kw["schedule"] = kernel
         ml = torch.full((rows, H, NP), float("nan"), dtype=torch.float32, device=dev)
         es = torch.full_like(ml, float("nan"))
         tmp = torch.full((rows, H, NP, D), float("nan"), dtype=torch.float32, device=dev)
@@ -199,6 +205,25 @@ def test_random_cases(oracle, seed):
     rng = random.Random(1000 + seed)
     for _ in range(CASES_PER_SEED):
         c = _draw_case(rng)
+        print(c, flush=True)
+        _run_case(oracle, c)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_single_head_groups_by_dot_products(oracle, seed):
+    """The shapes the dot-product kernels take (one query head per kv head, head size 128, fp16 queries, plain
+    decode) drawn like the other cases -- cache formats, layouts, block sizes, sinks, scales, empty and tiny
+    sequences -- through both of their schedules."""
+    rng = random.Random(9000 + seed)
+    for k in range(CASES_PER_SEED):
+        c = _draw_case(rng)
+        c.update(D=128, G=1, qdtype=torch.float16, feats={}, dot_schedules=(4, 5))
+        c["Hk"] = rng.choice([1, 2, 8, 32])
+        if k % 4 == 3:  # more items than work-groups stay resident, several per work-group
+            c["S"] = rng.randint(20, 60)
+            c["Hk"] = 32
+            c["lens"] = [rng.choice([0, rng.randint(1, 40), rng.randint(1, 700)]) for _ in range(c["S"])]
+            c["lens"][0] = max(c["lens"][0], 1)
         print(c, flush=True)
         _run_case(oracle, c)
 
