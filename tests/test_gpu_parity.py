@@ -201,6 +201,34 @@ def test_dot_product_kernel_for_single_head_groups(oracle, fp8):
         _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/fallback")
 
 
+def test_unknown_pool_size(oracle, monkeypatch):
+    """shape.num_pool_blocks = 0, as a caller passes who does not know how many blocks the pools hold: the
+    persistent kernels need the size (they request block ids before they know the lengths), so every
+    schedule runs a grid form, block-table columns past a context are never read and ids are not clamped.
+    The Python modules always know the size; the shape is edited on its way into the library."""
+    L = _cabi.load()
+    edited = []
+    for entry in ("fa_paged_attention_loop", "fa_paged_attention_reduce", "fa_paged_attention_fp8_loop",
+                  "fa_paged_attention_fp8_reduce"):
+        def without_pool_size(*args, _real=getattr(L, entry), _entry=entry):
+            args[-2]._obj.num_pool_blocks = 0   # the fa_paged_attention_shape behind byref()
+            edited.append(_entry)
+            return _real(*args)
+        monkeypatch.setattr(L, entry, without_pool_size)
+    lens = [1, 33, 700, 0, 1537, 2048]
+    for cfg, kernel, schedules in ((1, "loop", (0, 1, 4, 5)), (2, "loop", (0,)), (2, "reduce", (0, 1)),
+                                   (3, "fp8_loop", (0, 2, 4, 5)), (4, "fp8_reduce", (0, 1, 2))):
+        w = W.make_config(cfg, num_seqs=len(lens), pool_blocks=4096, lens=lens)
+        w.sinks = torch.linspace(-1, 2, w.num_heads).to(w.query.dtype)
+        # columns of the block table past a context hold ids no pool has: nobody may read them
+        for s, n in enumerate(lens):
+            w.block_tables[s, -(-n // w.block_size):] = 0x7FFFFFF0
+        for schedule in schedules:
+            bufs, _ = _run(w, kernel, schedule=schedule)
+            _check(bufs.out, w, oracle, f"{w.name}/{kernel}/unknown pool size, schedule {schedule}")
+    assert len(edited) >= 16 and len(set(edited)) == 4
+
+
 def test_lds_staged_kernel_full_size(oracle):
     """The LDS-staged grid kernel on the whole FP8 loop configuration, both layouts, and E4M3 bytes."""
     for kw in (dict(), dict(layout=W.TOKEN_MAJOR), dict(fp8_dtype=torch.float8_e4m3fn)):
