@@ -16,6 +16,11 @@
 // us): four wavefronts and every resident work-group (three or four per unit) 104.6 / 59.5, eight
 // wavefronts 104.6 / 56.4, four wavefronts and two work-groups per unit 102.4 / 56.4 -- and 101.6 / 55.3
 // for the matrix-core kernel of the same schedule, which therefore stays the library's choice.
+// Persistent loop kernel with eight wavefronts per work-group where a launch has work-groups for at most
+// half the compute units (0: four wavefronts always).
+#ifndef FA_PLOOP_WIDE
+#define FA_PLOOP_WIDE 1
+#endif
 #ifndef FA_VALU_WAVES
 #define FA_VALU_WAVES 4
 #endif
@@ -113,8 +118,22 @@ inline fa_status launch_paged_attn_loop_rows(void *out, const void *query, const
           groups = pairs >= 2 * (int64_t)resident ? resident : std::min<int64_t>(cus, pairs);
         }
       }
+      // Work-groups for at most half the compute units (a handful of sequences): the launch is bound by
+      // what the few wavefronts keep in flight, and the same items with eight wavefronts per work-group keep
+      // twice as much.  Measured with 1, 2 and 4 sequences of 32 heads (us, four -> eight wavefronts): byte
+      // cache 17.5 -> 16.3, 17.0 -> 15.9, 18.4 -> 17.4; 16-bit cache 30.2 -> 29.4, 28.9 -> 28.6, 32.2 ->
+      // 31.8.  With a work-group on every unit it is a wash or a loss (upstream's perf shape, 256 items:
+      // 34.3 -> 35.0 us, byte cache 20.1 -> 20.8), and with head size 64 as well.
+      int waves = PW;
+      if constexpr (HEAD_SIZE == 128) {
+        if (FA_PLOOP_WIDE && kernel == plain && 2 * groups <= cus) {  // (teams of two kv heads need a pair per unit)
+          kernel = paged_attn_loop_persistent_kernel<HEAD_SIZE, QT, KVF, 2 * PW, PersistentLoop<KV8>::occ,
+                                                     Pipeline<KV8>::tiles_per_chunk, false, KROW, 1>;
+          waves = 2 * PW;
+        }
+      }
       const dim3 grid((unsigned)groups);
-      FA_HIP_CHECK(timer.launch(kernel, grid, dim3(PW * 64), 0, p));
+      FA_HIP_CHECK(timer.launch(kernel, grid, dim3(waves * 64), 0, p));
     } else if (KV8 && HEAD_SIZE == 128 && !ext && !r.pair_heads && r.schedule == FA_SCHEDULE_GRID_LDS) {
       // grid form, K and V staged through LDS: one work-group of eight wavefronts per compute unit
       if constexpr (KV8 && HEAD_SIZE == 128) {

@@ -226,7 +226,7 @@ def test_unknown_pool_size(oracle, monkeypatch):
         for schedule in schedules:
             bufs, _ = _run(w, kernel, schedule=schedule)
             _check(bufs.out, w, oracle, f"{w.name}/{kernel}/unknown pool size, schedule {schedule}")
-    assert len(edited) >= 16 and len(set(edited)) == 4
+    assert len(edited) == 14 and len(set(edited)) == 4
 
 
 def test_lds_staged_kernel_full_size(oracle):
