@@ -297,7 +297,8 @@ def test_persistent_split_many_items_per_wavefront(oracle):
 
 
 def _segment_mark(word):
-    """Segment length that slot 1 of a row of max_logits tells (None: no mark there)."""
+    """Segment length in the low byte of a mark, as slot 1 of a row of max_logits holds one behind a segment of
+    two or more partitions (None: the word is no mark)."""
     bits = int(word.view(torch.int32).item()) & 0xFFFFFFFF
     return (bits & 0xFF) if (bits & 0xFFFFFF00) == 0x7FD3A600 else None
 
@@ -307,8 +308,8 @@ def test_segment_kernel_partials_lie_a_segment_apart(oracle, batch):
     """Batches that the split path works in segments of several partitions: the output matches the
     oracle, and the scratch arrays hold one partial per segment, in the slot of the segment's
     first partition -- the partials the kernel model gives for a partition size of one segment --
-    and, in slot 1 of max_logits of every row of two or more partitions, the mark by which the
-    reduce kernel learns the segment length."""
+    and, in slot 1 of max_logits of every row of two or more partitions, a mark (the reduce kernel takes marked
+    slots for covered ones; the mark's low byte tells the segment length)."""
     gen = torch.Generator().manual_seed(21)
     if batch == "many_short":     # many sequences per compute unit: most sequences are one segment
         S = 64
