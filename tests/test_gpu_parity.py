@@ -201,6 +201,21 @@ def test_dot_product_kernel_for_single_head_groups(oracle, fp8):
         _check(bufs.out, w, oracle, f"{w.name}/valu{schedule}/fallback")
 
 
+@pytest.mark.parametrize("shape", [(16, 128, True), (32, 64, True), (16, 64, False), (64, 128, True), (24, 128, True)],
+                         ids=lambda s: f"hk{s[0]}_d{s[1]}_{'fp8' if s[2] else 'kv16'}")
+def test_loop_items_listed_by_memory_stack(oracle, shape):
+    """Head-major pools whose per-head chunks are 1, 2 or 4 KiB: the persistent loop kernels list a sequence's kv
+    heads so that a work-group's XCC reads one memory stack (csrc/paged_attention_items.h: stack_affine_head).
+    Whatever the order, every (sequence, kv head) must come out right -- shapes on which the map permutes the
+    heads, one with a head count it does not take (24), several items per work-group and fewer than work-groups."""
+    hk, d, fp8 = shape
+    for S in (3, 40):
+        w = W.make_test_shaped(batch_size=S, nheads=hk, nheads_k=hk, d=d, seqlen_k=300, varlen=True, has_sinks=True,
+                               fp8=fp8, block_size=16, layout=W.HEAD_MAJOR, seed=S)
+        bufs, _ = _run(w, ("fp8_" if fp8 else "") + "loop")
+        _check(bufs.out, w, oracle, f"{w.name}/stack-affine item order")
+
+
 def test_unknown_pool_size(oracle, monkeypatch):
     """shape.num_pool_blocks = 0, as a caller passes who does not know how many blocks the pools hold: the
     persistent kernels need the size (they request block ids before they know the lengths), so every
