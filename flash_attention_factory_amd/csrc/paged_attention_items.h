@@ -28,35 +28,6 @@ __device__ __forceinline__ int snake_position(int nth, int groups, int group) {
   return nth * groups + ((nth & 1) ? groups - 1 - group : group);
 }
 
-// Which kv head the q-th of a sequence's items is.  Work-groups are handed to the XCCs in turn (work-group g
-// runs on XCC g mod 8) and consecutive positions of the item list are the kv heads of one sequence, so with a
-// multiple of eight kv heads XCC k gets positions k, k + 8, ... of every sequence.  In a pool whose blocks hold
-// the heads' chunks side by side, head h lies h * (bytes of a head's chunk) into a block.  The timings below fit a
-// memory that is dealt to its eight stacks in 4 KiB units, by address bits 12 to 14 (an inference from the
-// measurements, not a documented fact): position q takes the head for which those bits equal q mod 8, so that
-// every XCC reads one stack and every stack is read by one XCC.
-// Measured on the FP8 Llama-7B decode batch (32 heads, chunks of 2 KiB, so that heads in plain order put two stacks
-// on each pair of neighbouring XCCs): 53.8 -> 52.8 us, and the XCCs' mean finishing times 47.8-51.1 -> within
-// 1.5 us of each other; giving every XCC every stack (heads rotated by the sequence's number) 53.1 us.  With chunks
-// of 4 KiB (16-bit cache, head size 128, blocks of 16) plain order is that map already.  Heads whose chunks are
-// smaller than 1 KiB or larger than 4 KiB (upstream's layout, where a head's share of a block is one token row at
-// a time; large blocks) stay in plain order.  shift: log2(4 KiB / chunk), or -1 for plain order.
-#ifndef FA_ITEM_HEAD_AFFINE
-#define FA_ITEM_HEAD_AFFINE 1
-#endif
-__device__ __forceinline__ int stack_affine_shift(int64_t head_chunk_bytes, int heads) {
-  if (!FA_ITEM_HEAD_AFFINE || head_chunk_bytes < 1024 || head_chunk_bytes > 4096 ||
-      (head_chunk_bytes & (head_chunk_bytes - 1)) != 0)
-    return -1;
-  const int shift = head_chunk_bytes == 4096 ? 0 : head_chunk_bytes == 2048 ? 1 : 2;
-  return heads % (8 << shift) == 0 ? shift : -1;
-}
-__device__ __forceinline__ int stack_affine_head(int q, int shift) {
-  if (shift < 0) return q;
-  const int k = q & 7, a = q >> 3;
-  return ((a >> shift) << (shift + 3)) | (k << shift) | (a & ((1 << shift) - 1));
-}
-
 template <int TPC>
 struct LoopItems {
   static constexpr int kMaxSeqs = 128;
