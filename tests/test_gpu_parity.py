@@ -205,7 +205,7 @@ def test_dot_product_kernel_for_single_head_groups(oracle, fp8):
                          ids=lambda s: f"hk{s[0]}_d{s[1]}_{'fp8' if s[2] else 'kv16'}")
 def test_loop_items_listed_by_memory_stack(oracle, shape):
     """Head-major pools whose per-head chunks are 1, 2 or 4 KiB: the persistent loop kernels list a sequence's kv
-    heads so that a work-group's XCC reads one memory stack (csrc/paged_attention_items.h: stack_affine_head).
+    heads so that a work-group's XCC reads one memory stack (csrc/paged_attention_utils.h: stack_affine_head).
     Whatever the order, every (sequence, kv head) must come out right -- shapes on which the map permutes the
     heads, one with a head count it does not take (24), several items per work-group and fewer than work-groups."""
     hk, d, fp8 = shape

@@ -1,4 +1,4 @@
-"""The order in which the persistent loop kernels list a sequence's kv heads (csrc/paged_attention_items.h:
+"""The order in which the persistent loop kernels list a sequence's kv heads (csrc/paged_attention_utils.h:
 stack_affine_shift, stack_affine_head), restated on the host: whatever the pool, every head is listed exactly
 once, and where the map applies the q-th item's chunk lies in the 4 KiB units that go to memory stack q mod 8."""
 import pytest
